@@ -1,0 +1,466 @@
+// Mixture-of-experts feed-forward (gfx950) and the residual boundary of layers whose sublayers run side by side:
+//   * router: fp32 logits of a tile of tokens against all experts, softmax scores, group-limited choice of the
+//     best `top` experts per token (a group's score is its best expert's; only the `keep` best groups are open),
+//     the chosen scores as weights (not renormalised); an extra logit row gives the shared expert's sigmoid gate,
+//   * alignment: the (token, choice) pairs sorted by expert (counting sort in one workgroup),
+//   * grouped GEMMs over the sorted rows: gate | up with the SiLU unit fused, then down, written back in (token,
+//     choice) order,
+//   * boundary: x += mixer + shared * gate + sum_k weight_k expert_k in fp32, then the next RMS norm, one pass.
+// Activations are bf16 or fp32 (dt: 0 = bf16, 1 = fp32); logits, scores, weights and the residual are fp32 in both.
+#include "common.h"
+
+GRAG_ERR_UNIT(moe)
+
+namespace grag {
+
+template <typename T> __device__ __forceinline__ float ldm(const T* p);
+template <> __device__ __forceinline__ float ldm<bf16>(const bf16* p) { return (float)*p; }
+template <> __device__ __forceinline__ float ldm<float>(const float* p) { return *p; }
+template <typename T> __device__ __forceinline__ void stm(T* p, float v);
+template <> __device__ __forceinline__ void stm<bf16>(bf16* p, float v) { *p = (bf16)v; }
+template <> __device__ __forceinline__ void stm<float>(float* p, float v) { *p = v; }
+
+// ------------------------------------------------------------------------------------------------ router
+constexpr int RT_TOK = 16;    // tokens per workgroup
+constexpr int RT_KC = 32;     // columns of h / the router matrix staged per step
+constexpr int RT_MAXR = 256;  // logit rows (experts + the shared gate's row) at most
+constexpr int RT_MAXTOP = 16;
+
+// h [T][ld] (the normed layer input); wr [R][W] fp32, rows 0 .. E-1 the experts, row E (R = E + 1) the shared expert's
+// gate.  ids [T][top] int32, wts [T][top] fp32 (the chosen experts by falling score; ties to the lower index),
+// sgate [T] fp32 = sigmoid(row E's logit).  grid (ceil(T / RT_TOK)), 256 threads: thread (token tid % 16, part
+// tid / 16) owns logit rows part, part + 16, ...
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ wr, int W, int E, int R, int top,
+                 int ngroups, int keep, int* __restrict__ ids, float* __restrict__ wts, float* __restrict__ sgate,
+                 int T_) {
+  __shared__ float hs[RT_TOK][RT_KC + 1];
+  __shared__ float ws[RT_MAXR][RT_KC + 1];
+  __shared__ float lg[RT_TOK][RT_MAXR + 1];
+  const int tok = threadIdx.x & 15, part = threadIdx.x >> 4;
+  const int t0 = blockIdx.x * RT_TOK;
+  float acc[RT_MAXR / 16];
+#pragma unroll
+  for (int j = 0; j < RT_MAXR / 16; ++j) acc[j] = 0.f;
+  for (int k0 = 0; k0 < W; k0 += RT_KC) {
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < RT_TOK * RT_KC; idx += 256) {
+      const int tt = idx / RT_KC, k = idx - tt * RT_KC;
+      hs[tt][k] = (t0 + tt < T_ && k0 + k < W) ? ldm(h + (size_t)(t0 + tt) * ld + k0 + k) : 0.f;
+    }
+    for (int idx = threadIdx.x; idx < R * RT_KC; idx += 256) {
+      const int r = idx / RT_KC, k = idx - r * RT_KC;
+      ws[r][k] = k0 + k < W ? wr[(size_t)r * W + k0 + k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < RT_MAXR / 16; ++j) {
+      const int r = part + 16 * j;
+      if (r < R) {
+        float a = acc[j];
+#pragma unroll
+        for (int k = 0; k < RT_KC; ++k) a = fmaf(hs[tok][k], ws[r][k], a);
+        acc[j] = a;
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < RT_MAXR / 16; ++j)
+    if (part + 16 * j < R) lg[tok][part + 16 * j] = acc[j];
+  __syncthreads();
+  if (threadIdx.x >= RT_TOK || t0 + threadIdx.x >= T_) return;
+  float* z = lg[threadIdx.x];
+  const int t = t0 + threadIdx.x;
+  if (R > E && sgate != nullptr) sgate[t] = 1.f / (1.f + expf(-z[E]));
+  float mx = -INFINITY;
+  for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
+  float sum = 0.f;
+  for (int e = 0; e < E; ++e) sum += expf(z[e] - mx);
+  const float inv = 1.f / sum;
+  // the open groups: `keep` times, the best group not yet taken (by its best logit: softmax keeps the order)
+  const int per = E / ngroups;
+  unsigned long long open_lo = 0, open_hi = 0, open_2 = 0, open_3 = 0;  // bit g: group g is open (up to 256 groups)
+  auto is_open = [&](int g) {
+    const unsigned long long wbits = g < 64 ? open_lo : g < 128 ? open_hi : g < 192 ? open_2 : open_3;
+    return (wbits >> (g & 63)) & 1ull;
+  };
+  for (int n = 0; n < keep; ++n) {
+    int bg = -1;
+    float bv = -INFINITY;
+    for (int g = 0; g < ngroups; ++g) {
+      if (is_open(g)) continue;
+      float gv = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) gv = fmaxf(gv, z[e]);
+      if (bg < 0 || gv > bv) {
+        bg = g;
+        bv = gv;
+      }
+    }
+    if (bg < 0) break;
+    const unsigned long long bit = 1ull << (bg & 63);
+    if (bg < 64) open_lo |= bit;
+    else if (bg < 128) open_hi |= bit;
+    else if (bg < 192) open_2 |= bit;
+    else open_3 |= bit;
+  }
+  // the best `top` experts of the open groups; a taken expert's logit is overwritten with -inf
+  for (int n = 0; n < top; ++n) {
+    int be = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      if (!is_open(e / per)) continue;
+      const float v = z[e];
+      if (v > bv || (be < 0 && v > -INFINITY)) {
+        be = e;
+        bv = v;
+      }
+    }
+    if (be < 0) {  // fewer open experts than `top`: the rest of the choices carry no weight
+      ids[(size_t)t * top + n] = 0;
+      wts[(size_t)t * top + n] = 0.f;
+      continue;
+    }
+    ids[(size_t)t * top + n] = be;
+    wts[(size_t)t * top + n] = expf(bv - mx) * inv;
+    z[be] = -INFINITY;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ alignment
+// ids [n] (n = T * top) -> offs [E + 1] (rows of expert e are order[offs[e] .. offs[e + 1])) and order [n]: the flat
+// (token * top + choice) index of every sorted row.  One workgroup of 1024 threads; rows of one expert keep no
+// particular order (every row is computed on its own, the sums over a token's choices run in choice order later).
+__global__ void __launch_bounds__(1024)
+moe_align_kernel(const int* __restrict__ ids, int n, int E, int* __restrict__ offs, int* __restrict__ order) {
+  __shared__ int cnt[RT_MAXR];
+  __shared__ int pos[RT_MAXR];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int e = ids[i];
+    if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int s = 0;
+    for (int e = 0; e < E; ++e) {
+      offs[e] = s;
+      pos[e] = s;
+      s += cnt[e];
+    }
+    offs[E] = s;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int e = ids[i];
+    if (e >= 0 && e < E) order[atomicAdd(&pos[e], 1)] = i;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ grouped GEMM
+// Rows sorted by expert; the workgroup of row tile blockIdx.y finds its expert by walking offs (tiles never straddle
+// two experts).  GATED 1: A row r = h[order[r] / top] (gathered), B = wgu[e] ([2F][K]: gate rows, then up rows),
+// out[r][n] = silu(a . gate_n) * (a . up_n), out [rows][F] in sorted order.  GATED 0: A row r = act[r] (sorted order),
+// B = wd[e] ([N][K]), out[order[r]][n] = a . w_n: back in (token, choice) order.
+// Plain tiles: 32 rows x 64 columns per workgroup, K in steps of 32 through LDS, fp32 accumulation; thread (ty, tx) of
+// 16 x 16 owns rows ty, ty + 16 and columns tx, tx + 16, tx + 32, tx + 48.
+constexpr int MG_M = 32, MG_N = 64, MG_K = 32;
+
+template <typename T, int GATED>
+__global__ void __launch_bounds__(256)
+moe_gemm_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, const int* __restrict__ offs,
+                const int* __restrict__ order, int E, int top, int N, int K, T* __restrict__ out, int ldo) {
+  __shared__ float As[MG_M][MG_K + 1];
+  __shared__ float Bs[GATED ? 2 : 1][MG_N][MG_K + 1];
+  __shared__ int rows[MG_M];
+  // the expert and row range of this tile
+  int e = 0, tile = blockIdx.y, r0 = -1, rend = 0;
+  for (; e < E; ++e) {
+    const int b = offs[e], n = offs[e + 1] - b, nt = (n + MG_M - 1) / MG_M;
+    if (tile < nt) {
+      r0 = b + tile * MG_M;
+      rend = b + n;
+      break;
+    }
+    tile -= nt;
+  }
+  if (r0 < 0) return;
+  const int n0 = blockIdx.x * MG_N;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  if (threadIdx.x < MG_M) {
+    const int r = r0 + threadIdx.x;
+    rows[threadIdx.x] = r < rend ? (GATED ? order[r] / top : r) : -1;
+  }
+  const size_t wrows = GATED ? (size_t)2 * N : (size_t)N;
+  const T* we = w + (size_t)e * wrows * K;
+  float acc[GATED ? 2 : 1][2][4];
+#pragma unroll
+  for (int u = 0; u < (GATED ? 2 : 1); ++u)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[u][i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += MG_K) {
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < MG_M * MG_K; idx += 256) {
+      const int m = idx / MG_K, k = idx - m * MG_K;
+      const int src = rows[m];
+      As[m][k] = (src >= 0 && k0 + k < K) ? ldm(a + (size_t)src * lda + k0 + k) : 0.f;
+    }
+    for (int idx = threadIdx.x; idx < MG_N * MG_K; idx += 256) {
+      const int n = idx / MG_K, k = idx - n * MG_K;
+      const bool ok = n0 + n < N && k0 + k < K;
+      Bs[0][n][k] = ok ? ldm(we + (size_t)(n0 + n) * K + k0 + k) : 0.f;
+      if (GATED) Bs[GATED ? 1 : 0][n][k] = ok ? ldm(we + (size_t)(N + n0 + n) * K + k0 + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int k = 0; k < MG_K; ++k) {
+      const float a0 = As[ty][k], a1 = As[ty + 16][k];
+#pragma unroll
+      for (int u = 0; u < (GATED ? 2 : 1); ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float b = Bs[u][tx + 16 * j][k];
+          acc[u][0][j] = fmaf(a0, b, acc[u][0][j]);
+          acc[u][1][j] = fmaf(a1, b, acc[u][1][j]);
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = r0 + ty + 16 * i;
+    if (r >= rend) continue;
+    const size_t orow = GATED ? (size_t)r : (size_t)order[r];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx + 16 * j;
+      if (n >= N) continue;
+      float v = acc[0][i][j];
+      if (GATED) v = v / (1.f + expf(-v)) * acc[GATED ? 1 : 0][i][j];
+      stm(out + orow * ldo + n, v);
+    }
+  }
+}
+
+// The same on the matrix cores (bf16, K a multiple of 16): 4 waves, each 16 rows x 32 columns of a 32 x 64 tile
+// (wave w: rows 16 (w / 2), columns 32 (w % 2)), v_mfma_f32_16x16x16_bf16 over K steps of 32 staged through LDS as
+// bf16.  A fragment: lane holds A[row lane % 16][k = 4 (lane / 16) .. + 3]; B fragment: B[k = 4 (lane / 16) .. + 3]
+// [col lane % 16] = w[col][k ..]; C fragment: rows 4 (lane / 16) + i, column lane % 16.
+template <int GATED>
+__global__ void __launch_bounds__(256)
+moe_gemm_mfma_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, const int* __restrict__ offs,
+                     const int* __restrict__ order, int E, int top, int N, int K, bf16* __restrict__ out, int ldo) {
+  constexpr int KS = MG_K + 8;  // LDS row stride (elements): 80 bytes, 16-byte aligned rows
+  __shared__ __attribute__((aligned(16))) short As[MG_M][KS];
+  __shared__ __attribute__((aligned(16))) short Bs[GATED ? 2 : 1][MG_N][KS];
+  __shared__ int rows[MG_M];
+  int e = 0, tile = blockIdx.y, r0 = -1, rend = 0;
+  for (; e < E; ++e) {
+    const int b = offs[e], n = offs[e + 1] - b, nt = (n + MG_M - 1) / MG_M;
+    if (tile < nt) {
+      r0 = b + tile * MG_M;
+      rend = b + n;
+      break;
+    }
+    tile -= nt;
+  }
+  if (r0 < 0) return;
+  const int n0 = blockIdx.x * MG_N;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int ql = lane & 15, quad = lane >> 4;
+  const int wr = (wid >> 1) * 16, wc = (wid & 1) * 32;
+  if (threadIdx.x < MG_M) {
+    const int r = r0 + threadIdx.x;
+    rows[threadIdx.x] = r < rend ? (GATED ? order[r] / top : r) : -1;
+  }
+  const size_t wrows = GATED ? (size_t)2 * N : (size_t)N;
+  const bf16* we = w + (size_t)e * wrows * K;
+  f32x4_t acc[GATED ? 2 : 1][2];
+#pragma unroll
+  for (int u = 0; u < (GATED ? 2 : 1); ++u)
+#pragma unroll
+    for (int c = 0; c < 2; ++c) acc[u][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  __syncthreads();
+  // staging: thread t loads 8 bf16 (16 bytes): A 32 rows x 4 vectors = 128 threads; B 64 rows x 4 vectors = 256 threads
+  const int sr = threadIdx.x >> 2, sv = (threadIdx.x & 3) * 8;
+  for (int k0 = 0; k0 < K; k0 += MG_K) {
+    bf16x8_t av = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0}, bv0 = av, bv1 = av;
+    if (threadIdx.x < 128) {
+      const int src = rows[sr];
+      if (src >= 0 && k0 + sv < K) av = *reinterpret_cast<const bf16x8_t*>(a + (size_t)src * lda + k0 + sv);
+    }
+    if (n0 + sr < N && k0 + sv < K) {
+      bv0 = *reinterpret_cast<const bf16x8_t*>(we + (size_t)(n0 + sr) * K + k0 + sv);
+      if (GATED) bv1 = *reinterpret_cast<const bf16x8_t*>(we + (size_t)(N + n0 + sr) * K + k0 + sv);
+    }
+    __syncthreads();
+    if (threadIdx.x < 128) *reinterpret_cast<bf16x8_t*>(&As[sr][sv]) = av;
+    *reinterpret_cast<bf16x8_t*>(&Bs[0][sr][sv]) = bv0;
+    if (GATED) *reinterpret_cast<bf16x8_t*>(&Bs[GATED ? 1 : 0][sr][sv]) = bv1;
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < MG_K / 16; ++ks) {
+      const bf16x4_t af = *reinterpret_cast<const bf16x4_t*>(&As[wr + ql][ks * 16 + quad * 4]);
+#pragma unroll
+      for (int u = 0; u < (GATED ? 2 : 1); ++u)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          const bf16x4_t bf = *reinterpret_cast<const bf16x4_t*>(&Bs[u][wc + 16 * c + ql][ks * 16 + quad * 4]);
+          acc[u][c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(af, bf, acc[u][c], 0, 0, 0);
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + wr + 4 * quad + i;
+    if (r >= rend) continue;
+    const size_t orow = GATED ? (size_t)r : (size_t)order[r];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int n = n0 + wc + 16 * c + ql;
+      if (n >= N) continue;
+      float v = acc[0][c][i];
+      if (GATED) v = v / (1.f + expf(-v)) * acc[GATED ? 1 : 0][c][i];
+      out[orow * ldo + n] = (bf16)v;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ residual boundary
+// x [T][H] fp32, in place: x <- keep x + (a + bcoef_t b + sum_k ecoef_(t,k) e_(t,k)), every addend optional
+// (a, b [T][H]; e [T * K][H], ecoef [T * K]; bcoef [T], null: 1).  Then, each optional: raw [T][raw_ld] <- x in the
+// activation type, out [T][H] <- x / sqrt(mean(x^2) + eps) * w.  grid (T), 256 threads; a thread keeps its elements of
+// the row in registers between the sum of squares and the scaling (rows of up to 256 * RB_PER), or re-reads x.
+constexpr int RB_PER = 16;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+residual_rmsnorm_kernel(float* __restrict__ x, float keep, const T* __restrict__ a, const T* __restrict__ b,
+                        const float* __restrict__ bcoef, const T* __restrict__ e, const float* __restrict__ ecoef,
+                        int K, const float* __restrict__ w, float eps, T* __restrict__ out, T* __restrict__ raw,
+                        int raw_ld, int H) {
+  __shared__ float red[16];
+  const size_t t = blockIdx.x, row = t * H;
+  const float bc = b ? (bcoef ? bcoef[t] : 1.f) : 0.f;
+  float v[RB_PER];
+  float ss = 0.f;
+  const bool fits = H <= 256 * RB_PER;
+#pragma unroll
+  for (int u = 0; u < RB_PER; ++u) {
+    v[u] = 0.f;
+    if (!fits) break;
+    const int i = threadIdx.x + 256 * u;
+    if (i < H) {
+      float y = a ? ldm(a + row + i) : 0.f;
+      float f = b ? bc * ldm(b + row + i) : 0.f;
+      for (int k = 0; k < K; ++k) f = fmaf(ecoef[t * K + k], ldm(e + (t * K + k) * H + i), f);
+      y += f;
+      const float nx = keep != 0.f ? keep * x[row + i] + y : y;
+      x[row + i] = nx;
+      v[u] = nx;
+      ss = fmaf(nx, nx, ss);
+      if (raw) stm(raw + t * raw_ld + i, nx);
+    }
+  }
+  if (!fits) {
+    for (int i = threadIdx.x; i < H; i += 256) {
+      float y = a ? ldm(a + row + i) : 0.f;
+      float f = b ? bc * ldm(b + row + i) : 0.f;
+      for (int k = 0; k < K; ++k) f = fmaf(ecoef[t * K + k], ldm(e + (t * K + k) * H + i), f);
+      y += f;
+      const float nx = keep != 0.f ? keep * x[row + i] + y : y;
+      x[row + i] = nx;
+      ss = fmaf(nx, nx, ss);
+      if (raw) stm(raw + t * raw_ld + i, nx);
+    }
+  }
+  if (out == nullptr) return;
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)H + eps);
+  if (fits) {
+#pragma unroll
+    for (int u = 0; u < RB_PER; ++u) {
+      const int i = threadIdx.x + 256 * u;
+      if (i < H) stm(out + row + i, v[u] * r * w[i]);
+    }
+  } else {
+    for (int i = threadIdx.x; i < H; i += 256) stm(out + row + i, x[row + i] * r * w[i]);
+  }
+}
+
+}  // namespace grag
+
+using namespace grag;
+
+#define DT_DISPATCH(dt, ...)                   \
+  if ((dt) == 0) {                             \
+    using T = bf16;                            \
+    __VA_ARGS__                                \
+  } else {                                     \
+    using T = float;                           \
+    __VA_ARGS__                                \
+  }
+
+GRAG_API int grag_moe_max_rows() { return RT_MAXR; }
+GRAG_API int grag_moe_max_top() { return RT_MAXTOP; }
+
+GRAG_API hipError_t grag_moe_route(const void* h, int ld, const float* wr, int W, int E, int R, int top, int ngroups,
+                                   int keep, int* ids, float* wts, float* sgate, int T_, int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  if (E < 1 || R < E || R > RT_MAXR || top < 1 || top > RT_MAXTOP || top > E || ngroups < 1 || E % ngroups ||
+      keep < 1 || keep > ngroups)
+    return hipErrorInvalidValue;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(moe_route_kernel<T>, dim3((T_ + RT_TOK - 1) / RT_TOK), dim3(256), 0, st,
+                                     (const T*)h, ld, wr, W, E, R, top, ngroups, keep, ids, wts, sgate, T_);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_moe_align(const int* ids, int n, int E, int* offs, int* order, hipStream_t st) {
+  if (n <= 0) return hipSuccess;
+  if (E < 1 || E > RT_MAXR) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), 0, st, ids, n, E, offs, order);
+  return hipGetLastError();
+}
+
+// rows = T * top sorted rows.  gated 1: a = h [T][lda], w = [E][2N][K], out [rows][N]; gated 0: a = [rows][lda] sorted,
+// w = [E][N][K], out [rows][ldo] in (token, choice) order.
+GRAG_API hipError_t grag_moe_gemm(const void* a, int lda, const void* w, const int* offs, const int* order, int rows,
+                                  int E, int top, int N, int K, void* out, int ldo, int gated, int dt, hipStream_t st) {
+  if (rows <= 0) return hipSuccess;
+  const int tiles = (rows + MG_M - 1) / MG_M + E;  // every expert may end on a partial tile
+  if (tiles > 65535 || E < 1 || top < 1) return hipErrorInvalidValue;
+  const dim3 grid((N + MG_N - 1) / MG_N, tiles);
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (dt == 0 && K % 8 == 0 && lda % 8 == 0 && al16(a) && al16(w)) {
+    if (gated)
+      hipLaunchKernelGGL(moe_gemm_mfma_kernel<1>, grid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,
+                         order, E, top, N, K, (bf16*)out, ldo);
+    else
+      hipLaunchKernelGGL(moe_gemm_mfma_kernel<0>, grid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,
+                         order, E, top, N, K, (bf16*)out, ldo);
+    return hipGetLastError();
+  }
+  DT_DISPATCH(dt, {
+    if (gated)
+      hipLaunchKernelGGL((moe_gemm_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)a, lda, (const T*)w, offs, order, E,
+                         top, N, K, (T*)out, ldo);
+    else
+      hipLaunchKernelGGL((moe_gemm_kernel<T, 0>), grid, dim3(256), 0, st, (const T*)a, lda, (const T*)w, offs, order, E,
+                         top, N, K, (T*)out, ldo);
+  })
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_residual_rmsnorm(float* x, float keep, const void* a, const void* b, const float* bcoef,
+                                          const void* e, const float* ecoef, int K, const float* w, float eps,
+                                          void* out, void* raw, int raw_ld, int T_, int H, int dt, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  if (K < 0 || (K > 0 && (e == nullptr || ecoef == nullptr)) || (out != nullptr && w == nullptr))
+    return hipErrorInvalidValue;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(residual_rmsnorm_kernel<T>, dim3(T_), dim3(256), 0, st, x, keep, (const T*)a,
+                                     (const T*)b, bcoef, (const T*)e, ecoef, e ? K : 0, w, eps, (T*)out, (T*)raw,
+                                     raw_ld, H);)
+  return hipGetLastError();
+}

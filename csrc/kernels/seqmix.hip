@@ -103,14 +103,16 @@ __global__ void dyt_residual_vec_kernel(const T* __restrict__ y, float a1, const
 // ------------------------------------------------------------------------------------------------ rotary + K/V store
 // proj [T, ld]: q heads at column qoff (H x d), k heads at koff (G x d), v heads at voff (G x vd).
 // q_out [T, H*d] = rotated q; k_cache [nblk, G, BS, d] <- rotated k; v_cache [nblk, G, BS, vd] <- v / rms(v).
-// Rotation: the first rd dims of a head, dim i paired with i + rd/2; table row p = cos[0:rd/2] | sin[0:rd/2] (fp32).
+// Rotation: the first rd dims of a head, dim i paired with i + rd/2 (flags bit 0 set: dim 2i paired with 2i + 1, the
+// interleaved layout); table row p = cos[0:rd/2] | sin[0:rd/2] (fp32).  flags bit 1 set: the values are stored as
+// they are (no RMS division).
 // grid (T, ceil((H + G + G) / 4)), 256 threads: one wave per (token, head): q heads, then k heads, then v heads.
 template <typename T>
 __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int qoff, int koff, int voff,
                                         const int* __restrict__ positions, const float* __restrict__ table,
                                         int table_rows, const int* __restrict__ slot_mapping, T* __restrict__ q_out,
                                         T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int d, int vd,
-                                        int rd, int BS, long nslots, float eps) {
+                                        int rd, int BS, long nslots, float eps, int flags) {
   const int t = blockIdx.x, hb = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (hb >= H + 2 * G) return;
   const T* row = proj + (size_t)t * ld;
@@ -126,7 +128,7 @@ __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int 
       ss += v * v;
     }
     ss = wave_sum(ss);
-    const float r = 1.f / sqrtf(ss / (float)vd + eps);
+    const float r = (flags & 2) ? 1.f : 1.f / sqrtf(ss / (float)vd + eps);
     if (store)
       for (int i = lane; i < vd; i += 64) stf(v_cache + (((size_t)blk * G + g) * BS + off) * vd + i, ldf(x + i) * r);
     return;
@@ -142,7 +144,10 @@ __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int 
   T* dst = isq ? q_out + ((size_t)t * H + hh) * d : k_cache + (((size_t)blk * G + hh) * BS + off) * d;
   for (int i = lane; i < d; i += 64) {
     float v = ldf(x + i);
-    if (i < rd && pos_ok) {
+    if (i < rd && pos_ok && (flags & 1)) {  // adjacent pairs: (2j, 2j + 1) turned by angle j
+      const int j = i >> 1;
+      v = (i & 1) ? v * cs[j] + ldf(x + i - 1) * cs[half + j] : v * cs[j] - ldf(x + i + 1) * cs[half + j];
+    } else if (i < rd && pos_ok) {
       if (i < half) {
         v = v * cs[i] - ldf(x + i + half) * cs[half + i];
       } else {
@@ -157,6 +162,24 @@ __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int 
 // ------------------------------------------------------------------------------------------------ sink attention
 // softmax over the visible keys plus one key-less, value-less term exp(sink_h) in the denominator: the running
 // (max, sum) starts at (sink_h, 1) instead of (-inf, 0).
+// Optional extras (AttnExtra, all off when zero): `hscale` [H] multiplies the score scale of head h (a temperature per
+// head); `chunk` > 0 confines a query at position i to the keys j of its own aligned block of `chunk` positions,
+// floor(j / chunk) == floor(i / chunk) (and j <= i); `hgate` [T][gate_ld] holds one logit per (token, head) and the
+// head's output is multiplied by its sigmoid as it is stored.
+struct AttnExtra {
+  const float* hscale;
+  const void* hgate;
+  int gate_ld;
+  int chunk;
+};
+template <typename T>
+__device__ __forceinline__ float head_gate(const AttnExtra& ex, size_t row, int h) {
+  return ex.hgate ? sigmoid_acc(ldf(reinterpret_cast<const T*>(ex.hgate) + row * ex.gate_ld + h)) : 1.f;
+}
+__device__ __forceinline__ int chunk_start(const AttnExtra& ex, int pos) {
+  return ex.chunk > 0 ? pos - pos % ex.chunk : 0;
+}
+
 constexpr int SA_NQ = 4;   // queries per wave (prefill)
 constexpr int SA_VC = 8;   // 64-wide value-dim chunks per lane: vd <= 512 (a latent cache's value row can be that wide)
 
@@ -168,7 +191,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
                          T* __restrict__ out, int out_ld, const int* __restrict__ block_tables, int bt_stride,
                          const int* __restrict__ q_start, const int* __restrict__ ctx_len,
                          const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
-                         float out_scale, int KT, int nblocks, int v_ld) {
+                         float out_scale, int KT, int nblocks, int v_ld, AttnExtra ex) {
   extern __shared__ float smem[];
   const int QT = 4 * SA_NQ;
   const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
@@ -187,6 +210,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
     Qs[idx] = tq < qlen ? ldf(q + ((size_t)(qa + tq) * H + h) * d + i) : 0.f;
   }
   const int pos0 = ctx - qlen;  // position of the launch's first query of this sequence
+  if (ex.hscale) scale *= ex.hscale[h];
   float m[SA_NQ], l[SA_NQ], acc[SA_NQ][SA_VC];
   const float sink = sinks[h];
 #pragma unroll
@@ -199,7 +223,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
   const int last_q = min(q0 + QT, qlen) - 1;
   const int nkeys = min(ctx, pos0 + last_q + 1);
   const int* bt = block_tables + (size_t)seq * bt_stride;
-  for (int k0 = 0; k0 < nkeys; k0 += KT) {
+  for (int k0 = chunk_start(ex, pos0 + q0); k0 < nkeys; k0 += KT) {  // (the tile's first query has the earliest block)
     __syncthreads();
     const int kn = min(KT, nkeys - k0);
     for (int idx = threadIdx.x; idx < kn * d; idx += 256) {
@@ -237,7 +261,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
 #pragma unroll
     for (int n = 0; n < SA_NQ; ++n) {
       const int tq = q0 + wid * SA_NQ + n;
-      const bool vis = lane < kn && tq < qlen && (k0 + lane) <= pos0 + tq;
+      const bool vis = lane < kn && tq < qlen && (k0 + lane) <= pos0 + tq && (k0 + lane) >= chunk_start(ex, pos0 + tq);
       const float sc = vis ? s[n] * scale : -INFINITY;
       const float mn = fmaxf(m[n], wave_max(sc));
       const float p = vis ? expf(sc - mn) : 0.f;
@@ -268,7 +292,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
   for (int n = 0; n < SA_NQ; ++n) {
     const int tq = q0 + wid * SA_NQ + n;
     if (tq >= qlen) continue;
-    const float r = out_scale / l[n];
+    const float r = out_scale / l[n] * head_gate<T>(ex, (size_t)(qa + tq), h);
 #pragma unroll
     for (int c = 0; c < SA_VC; ++c) {
       const int j = lane + 64 * c;
@@ -292,7 +316,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
                               const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
                               const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ q_start,
                               const int* __restrict__ ctx_len, const float* __restrict__ sinks, int H, int G, int d,
-                              int vd, int BS, float scale, float out_scale, int nblocks, int v_ld) {
+                              int vd, int BS, float scale, float out_scale, int nblocks, int v_ld, AttnExtra ex) {
   constexpr int KT = 64;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   const int seq = blockIdx.z, h = blockIdx.y, g = h / (H / G);
@@ -324,23 +348,28 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
   const int qpos = pos0 + tq;
   // scores are kept in the log2 domain (one multiply by scale * log2 e, then v_exp_f32): m is the running max there
   const float LOG2E = 1.4426950408889634f;
-  const float sc2 = scale * LOG2E;
+  const float sc2 = scale * (ex.hscale ? ex.hscale[h] : 1.f) * LOG2E;
   float m = sinks[h] * LOG2E, l = 1.f;
   f32x4_t acc[NVM];
 #pragma unroll
   for (int v = 0; v < NVM; ++v) acc[v] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const int nkeys = min(ctx, pos0 + min(q0 + 64, qlen));
   const int wave_qmax = pos0 + min(q0 + wid * 16 + 15, qlen - 1);
+  // aligned blocks of ex.chunk positions: the tile loop starts at the block of the workgroup's first query; a wave skips
+  // the tiles before the block of ITS first query, and masks against each query's own block start
+  const int kfirst = chunk_start(ex, pos0 + q0);
+  const int wave_cmin = chunk_start(ex, pos0 + q0 + wid * 16), wave_cmax = chunk_start(ex, wave_qmax);
+  const int cstart = chunk_start(ex, q_ok ? qpos : pos0 + q0);
   const int* bt = block_tables + (size_t)seq * bt_stride;
   bf16x8_t kreg[NKM / 2], vreg[NVM / 2];
   RowCursor rc;
-  rc.init(threadIdx.x >> 2, BS);
+  rc.init(kfirst + (threadIdx.x >> 2), BS);
   {
-    const int blk = tile_block(rc, bt, threadIdx.x >> 2, nkeys, nblocks, ERR_BLOCK_PREFILL);
+    const int blk = tile_block(rc, bt, kfirst + (threadIdx.x >> 2), nkeys, nblocks, ERR_BLOCK_PREFILL);
     tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
     tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS, v_ld);
   }
-  for (int k0 = 0; k0 < nkeys; k0 += KT) {
+  for (int k0 = kfirst; k0 < nkeys; k0 += KT) {
     __syncthreads();
     tile_store(kreg, Ks, d, kstride);
     tile_store_v4(vreg, Vs, vd, vstride);
@@ -351,7 +380,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
       tile_load(kreg, k_cache, blk, rc.off, d, G, g, BS);
       tile_load(vreg, v_cache, blk, rc.off, vd, G, g, BS, v_ld);
     }
-    if (k0 > wave_qmax) continue;  // every key of the tile lies after this wave's queries
+    if (k0 > wave_qmax || k0 + KT <= wave_cmin) continue;  // every key lies after, or in a block before, this wave's queries
     f32x4_t st[4];
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
@@ -371,7 +400,8 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
     }
     float tmax = -INFINITY;
     // a tile wholly at or before the wave's first query (and inside the context) needs no mask
-    const bool interior = k0 + KT - 1 <= pos0 + q0 + wid * 16 && k0 + KT <= nkeys && q0 + wid * 16 + 15 < qlen;
+    const bool interior = k0 + KT - 1 <= pos0 + q0 + wid * 16 && k0 + KT <= nkeys && q0 + wid * 16 + 15 < qlen &&
+                          k0 >= wave_cmax;
     if (interior) {
 #pragma unroll
       for (int n = 0; n < 4; ++n)
@@ -386,7 +416,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = k0 + 16 * n + 4 * quad + i;
-          const bool vis = q_ok && key < nkeys && key <= qpos;
+          const bool vis = q_ok && key < nkeys && key <= qpos && key >= cstart;
           st[n][i] = vis ? st[n][i] * sc2 : -INFINITY;
           tmax = fmaxf(tmax, st[n][i]);
         }
@@ -447,7 +477,7 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
     const float li = __shfl(l, 4 * quad + i, 64);
     const int tr = q0 + wid * 16 + 4 * quad + i;  // the query of accumulator row i
     if (tr < qlen) {
-      const float r = out_scale / li;
+      const float r = out_scale / li * head_gate<bf16>(ex, (size_t)(qa + tr), h);
       bf16* orow = out + (size_t)(qa + tr) * out_ld + h * vd + ql;
 #pragma unroll
       for (int v = 0; v < NVM; ++v)
@@ -476,7 +506,7 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
                              const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
                              float out_scale, int nblocks, int nsplit, int split_len, float* __restrict__ part_o,
                              float* __restrict__ part_ml, int window, const bf16* __restrict__ gate, int gate_ld,
-                             int v_ld) {
+                             int v_ld, AttnExtra ex) {
   constexpr int KT = 64;
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   const int R = H / G, ngrp = (R + 15) >> 4;
@@ -499,13 +529,14 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
       qf[ks] = *reinterpret_cast<const bf16x4_t*>(q + ((size_t)seq * H + head) * d + ks * 16 + quad * 4);
   }
   const bool has_sink = !SIG && sp == 0 && wid == 0;
+  if (!SIG && ex.hscale) scale *= ex.hscale[head];  // (a fragment column is a head: one scale per lane)
   float m = has_sink ? sinks[head] : -INFINITY, l = has_sink ? 1.f : 0.f;
   const float pb = SIG ? sinks[head] : 0.f;
   f32x4_t acc[NVM];
 #pragma unroll
   for (int v = 0; v < NVM; ++v) acc[v] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const int kbeg = SIG ? max(0, ctx - window) : nsplit > 1 ? sp * split_len : 0;
-  const int kend = SIG ? ctx : nsplit > 1 ? min(ctx, kbeg + split_len) : ctx;
+  const int kend = SIG ? ctx : nsplit > 1 ? min(ctx, sp * split_len + split_len) : ctx;
+  const int kbeg = SIG ? max(0, ctx - window) : max(nsplit > 1 ? sp * split_len : 0, chunk_start(ex, ctx - 1));
   const int* bt = block_tables + (size_t)seq * bt_stride;
   bf16x8_t kreg[NKM / 2], vreg[NVM / 2];
   RowCursor rc;
@@ -640,7 +671,8 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
         if (!SIG && nsplit > 1) {
           part_o[(((size_t)sp * nseq + seq) * H + hr) * vd + 16 * v + ql] = x;
         } else {
-          const float gt = (SIG && gate) ? sigmoid_acc((float)gate[(size_t)seq * gate_ld + hr * vd + 16 * v + ql]) : 1.f;
+          const float gt = (SIG && gate) ? sigmoid_acc((float)gate[(size_t)seq * gate_ld + hr * vd + 16 * v + ql])
+                                         : SIG ? 1.f : head_gate<bf16>(ex, (size_t)seq, hr);
           out[(size_t)seq * out_ld + hr * vd + 16 * v + ql] = (bf16)(x * (out_scale / Lr) * gt);
         }
       }
@@ -651,7 +683,7 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
 // out = out_scale * sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the key splits; grid (H, nseq).
 __global__ void sink_attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                          bf16* __restrict__ out, int out_ld, int nsplit, int nseq, int H, int vd,
-                                         float out_scale) {
+                                         float out_scale, AttnExtra ex) {
   const int h = blockIdx.x, seq = blockIdx.y;
   float M = -INFINITY;
   for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(((size_t)s * nseq + seq) * H + h) * 2]);
@@ -660,7 +692,7 @@ __global__ void sink_attn_combine_kernel(const float* __restrict__ part_o, const
     const float* ml = part_ml + (((size_t)s * nseq + seq) * H + h) * 2;
     L += ml[0] == -INFINITY ? 0.f : ml[1] * expf(ml[0] - M);
   }
-  const float r = out_scale / L;
+  const float r = out_scale / L * head_gate<bf16>(ex, (size_t)seq, h);
   for (int j = threadIdx.x; j < vd; j += blockDim.x) {
     float o = 0.f;
     for (int s = 0; s < nsplit; ++s) {
@@ -678,10 +710,12 @@ sink_attn_decode_vec_kernel(const bf16* __restrict__ q, const bf16* __restrict__
                             const bf16* __restrict__ v_cache, bf16* __restrict__ out, int out_ld,
                             const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ ctx_len,
                             const float* __restrict__ sinks, int H, int G, int d, int vd, int BS, float scale,
-                            float out_scale, int nblocks, int v_ld) {
+                            float out_scale, int nblocks, int v_ld, AttnExtra ex) {
   extern __shared__ float smem[];
   const int seq = blockIdx.y, h = blockIdx.x, g = h / (H / G);
   const int ctx = ctx_len[seq];
+  const int kbeg = chunk_start(ex, ctx - 1);
+  if (ex.hscale) scale *= ex.hscale[h];
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   float* Qs = smem;               // [d]
   float* Ps = Qs + d;             // [4][64]
@@ -698,9 +732,9 @@ sink_attn_decode_vec_kernel(const bf16* __restrict__ q, const bf16* __restrict__
   float* pw = Ps + wid * 64;
   const int ntiles = (ctx + 63) >> 6;
   const int d8 = d >> 3;
-  for (int t = wid; t < ntiles; t += 4) {
+  for (int t = (kbeg >> 6) + wid; t < ntiles; t += 4) {
     const int key = t * 64 + lane;
-    const bool vis = key < ctx;
+    const bool vis = key < ctx && key >= kbeg;
     float s = 0.f;
     if (vis) {
       int blk = bt[key / BS];
@@ -728,7 +762,7 @@ sink_attn_decode_vec_kernel(const bf16* __restrict__ q, const bf16* __restrict__
       const int j = 2 * lane + 128 * c;
       float a0 = acc[c][0] * alpha, a1 = acc[c][1] * alpha;
       if (j < vd) {
-        for (int kk = 0; kk < kn; ++kk) {
+        for (int kk = max(0, kbeg - t * 64); kk < kn; ++kk) {
           const int key2 = t * 64 + kk;
           int b2 = bt[key2 / BS];
           if (b2 < 0 || b2 >= nblocks) b2 = 0;
@@ -764,7 +798,7 @@ sink_attn_decode_vec_kernel(const bf16* __restrict__ q, const bf16* __restrict__
       f[w] = Ms[w] == -INFINITY ? 0.f : expf(Ms[w] - M);
       L += Ms[4 + w] * f[w];
     }
-    const float r = out_scale / L;
+    const float r = out_scale / L * head_gate<bf16>(ex, (size_t)seq, h);
     for (int j = lane; j < vd; j += 64) {
       float o = 0.f;
       for (int w = 0; w < 4; ++w) o += As[w * vd + j] * f[w];
@@ -780,10 +814,12 @@ __global__ void __launch_bounds__(256)
 sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                         T* __restrict__ out, int out_ld, const int* __restrict__ block_tables, int bt_stride,
                         const int* __restrict__ ctx_len, const float* __restrict__ sinks, int H, int G, int d, int vd,
-                        int BS, float scale, float out_scale, int nblocks, int v_ld) {
+                        int BS, float scale, float out_scale, int nblocks, int v_ld, AttnExtra ex) {
   extern __shared__ float smem[];
   const int seq = blockIdx.y, h = blockIdx.x, g = h / (H / G);
   const int ctx = ctx_len[seq];
+  const int kbeg = chunk_start(ex, ctx - 1);
+  if (ex.hscale) scale *= ex.hscale[h];
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   float* Qs = smem;               // [d]
   float* Ps = Qs + d;             // [4][64]
@@ -798,9 +834,9 @@ sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, 
   const int* bt = block_tables + (size_t)seq * bt_stride;
   float* pw = Ps + wid * 64;
   const int ntiles = (ctx + 63) >> 6;
-  for (int t = wid; t < ntiles; t += 4) {
+  for (int t = (kbeg >> 6) + wid; t < ntiles; t += 4) {
     const int key = t * 64 + lane;
-    const bool vis = key < ctx;
+    const bool vis = key < ctx && key >= kbeg;
     float s = 0.f;
     int blk = 0;
     if (vis) {
@@ -825,7 +861,7 @@ sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, 
       const int j = lane + 64 * c;
       float a = acc[c] * alpha;
       if (j < vd) {
-        for (int kk = 0; kk < kn; ++kk) {
+        for (int kk = max(0, kbeg - t * 64); kk < kn; ++kk) {
           const int key2 = t * 64 + kk;
           int b2 = bt[key2 / BS];
           if (b2 < 0 || b2 >= nblocks) b2 = 0;
@@ -854,7 +890,7 @@ sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, 
       f[w] = Ms[w] == -INFINITY ? 0.f : expf(Ms[w] - M);
       L += Ms[4 + w] * f[w];
     }
-    const float r = out_scale / L;
+    const float r = out_scale / L * head_gate<T>(ex, (size_t)seq, h);
 #pragma unroll
     for (int c = 0; c < SA_VC; ++c) {
       const int j = lane + 64 * c;
@@ -1021,7 +1057,8 @@ __global__ void decay_chunk_prefix_kernel(const float* __restrict__ decay, float
 
 // out [T, out_ld slice] = out_scale * x / rms(x) * w * gate(g), x fp32 [T, groups * N] normalised per group of N
 // columns (grid (T, groups): the whole row, or one head at a time); w may be null (no weight); g at proj column
-// goff, gate = sigmoid (silu_gate 0) or SiLU (1).
+// goff, gate = sigmoid (silu_gate bit 0 clear) or SiLU (set).  silu_gate bit 1 set: the gate comes BEFORE the norm,
+// out = out_scale * u / rms(u) * w with u = x * gate(g).
 template <typename T>
 __global__ void gated_rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                      const T* __restrict__ proj, int ld, int goff, T* __restrict__ out, int out_ld,
@@ -1029,13 +1066,21 @@ __global__ void gated_rmsnorm_kernel(const float* __restrict__ x, const float* _
   __shared__ float red[16];
   const int t = blockIdx.x, c0 = blockIdx.y * N;
   const float* xr = x + (size_t)t * N * gridDim.y + c0;
+  const bool first = silu_gate & 2;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < N; i += blockDim.x) ss += xr[i] * xr[i];
+  for (int i = threadIdx.x; i < N; i += blockDim.x) {
+    float v = xr[i];
+    if (first) {
+      const float g = ldf(proj + (size_t)t * ld + goff + c0 + i);
+      v *= (silu_gate & 1) ? silu_acc(g) : sigmoid_acc(g);
+    }
+    ss += v * v;
+  }
   ss = block_sum(ss, red);
   const float r = out_scale / sqrtf(ss / (float)N + eps);
   for (int i = threadIdx.x; i < N; i += blockDim.x) {
     const float g = ldf(proj + (size_t)t * ld + goff + c0 + i);
-    const float gt = silu_gate ? silu_acc(g) : sigmoid_acc(g);
+    const float gt = (silu_gate & 1) ? silu_acc(g) : sigmoid_acc(g);
     stf(out + (size_t)t * out_ld + c0 + i, xr[i] * r * (w ? w[c0 + i] : 1.f) * gt);
   }
 }
@@ -1051,24 +1096,24 @@ gated_rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__
   if (grp >= groups) return;
   const int c0 = grp * N;
   const float* xr = x + (size_t)t * N * groups + c0;
-  float v[8];
+  const bool first = silu_gate & 2;
+  float v[8], gt[8];
   float ss = 0.f;
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     const int i = lane + 64 * k;
     v[k] = i < N ? xr[i] : 0.f;
-    ss = fmaf(v[k], v[k], ss);
+    const float g = i < N ? ldf(proj + (size_t)t * ld + goff + c0 + i) : 0.f;
+    gt[k] = (silu_gate & 1) ? silu_acc(g) : sigmoid_acc(g);
+    const float u = first ? v[k] * gt[k] : v[k];
+    ss = fmaf(u, u, ss);
   }
   ss = wave_sum(ss);
   const float r = out_scale / sqrtf(ss / (float)N + eps);
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     const int i = lane + 64 * k;
-    if (i < N) {
-      const float g = ldf(proj + (size_t)t * ld + goff + c0 + i);
-      const float gt = silu_gate ? silu_acc(g) : sigmoid_acc(g);
-      stf(out + (size_t)t * out_ld + c0 + i, v[k] * r * (w ? w[c0 + i] : 1.f) * gt);
-    }
+    if (i < N) stf(out + (size_t)t * out_ld + c0 + i, v[k] * r * (w ? w[c0 + i] : 1.f) * gt[k]);
   }
 }
 
@@ -1219,12 +1264,12 @@ GRAG_API hipError_t grag_dyt_residual(const void* y, float a1, const float* w1, 
 GRAG_API hipError_t grag_rope_vnorm_store(const void* proj, int ld, int qoff, int koff, int voff, const int* positions,
                                           const float* table, int table_rows, const int* slot_mapping, void* q_out,
                                           void* k_cache, void* v_cache, int T_, int H, int G, int d, int vd, int rd,
-                                          int BS, long nslots, float eps, int dt, hipStream_t st) {
+                                          int BS, long nslots, float eps, int dt, int flags, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
   if (H + 2 * G > 4 * 65535) return hipErrorInvalidValue;
   DT_DISPATCH(dt, hipLaunchKernelGGL(rope_vnorm_store_kernel<T>, dim3(T_, (H + 2 * G + 3) / 4), dim3(256), 0, st, (const T*)proj, ld, qoff,
                                      koff, voff, positions, table, table_rows, slot_mapping, (T*)q_out, (T*)k_cache,
-                                     (T*)v_cache, H, G, d, vd, rd, BS, nslots, eps);)
+                                     (T*)v_cache, H, G, d, vd, rd, BS, nslots, eps, flags);)
   return hipGetLastError();
 }
 
@@ -1244,7 +1289,9 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
                                            int out_ld, const int* block_tables, int bt_stride, const int* q_start,
                                            const int* ctx_len, const float* sinks, int nseq, int max_q_len, int H,
                                            int G, int d, int vd, int BS, float scale, float out_scale, int nblocks,
-                                           int dt, int v_ld, hipStream_t st) {
+                                           int dt, int v_ld, const float* hscale, const void* hgate, int gate_ld,
+                                           int chunk, hipStream_t st) {
+  const AttnExtra ex{hscale, hgate, gate_ld, chunk};
   // v_ld: elements from one cached value row to the next (vd, or more when the value rows are the head of wider rows)
   if (nseq <= 0 || max_q_len <= 0) return hipSuccess;
   if (vd > 64 * SA_VC || G <= 0 || H % G || v_ld < vd) return hipErrorInvalidValue;
@@ -1261,7 +1308,7 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
     }                                                                                                                \
     hipLaunchKernelGGL((sink_attn_prefill_mfma_kernel<NK, NV>), mgrid, dim3(256), mb, st, (const bf16*)q,            \
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
-                       q_start, ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld);                   \
+                       q_start, ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld, ex);               \
   }
     const int nk = d / 16, nv = vd / 16;
     if (nk <= 4 && nv <= 4) SA_MFMA(4, 4)
@@ -1284,7 +1331,7 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
     }
     hipLaunchKernelGGL(sink_attn_prefill_kernel<T>, grid, dim3(256), bytes, st, (const T*)q, (const T*)k_cache,
                        (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride, q_start, ctx_len, sinks, H, G, d,
-                       vd, BS, scale, out_scale, KT, nblocks, v_ld);
+                       vd, BS, scale, out_scale, KT, nblocks, v_ld, ex);
   })
   return hipGetLastError();
 }
@@ -1295,7 +1342,9 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
                                           int out_ld, const int* block_tables, int bt_stride, const int* ctx_len,
                                           const float* sinks, int nseq, int H, int G, int d, int vd, int BS,
                                           float scale, float out_scale, int nblocks, int dt, int nsplit,
-                                          int split_len, float* part_o, float* part_ml, int v_ld, hipStream_t st) {
+                                          int split_len, float* part_o, float* part_ml, int v_ld, const float* hscale,
+                                          const void* hgate, int gate_ld, int chunk, hipStream_t st) {
+  const AttnExtra ex{hscale, hgate, gate_ld, chunk};
   if (nseq <= 0) return hipSuccess;
   if (vd > 64 * SA_VC || G <= 0 || H % G || v_ld < vd) return hipErrorInvalidValue;
   if (dt == 0 && v_ld % 8 == 0 && (reinterpret_cast<uintptr_t>(v_cache) & 15) == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && G * ((H / G + 15) / 16) <= 65535 &&
@@ -1316,7 +1365,7 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
     hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV, 0>), mgrid, dim3(256), mb, st, (const bf16*)q,          \
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
                        ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, nsplit, split_len, part_o,        \
-                       part_ml, 0, (const bf16*)nullptr, 0, v_ld);                                                   \
+                       part_ml, 0, (const bf16*)nullptr, 0, v_ld, ex);                                               \
   }
     const int nk = d / 16, nv = vd / 16;
     if (nk <= 4 && nv <= 4) SD_MFMA(4, 4)
@@ -1327,19 +1376,19 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
 #undef SD_MFMA
     if (nsplit > 1)
       hipLaunchKernelGGL(sink_attn_combine_kernel, dim3(H, nseq), dim3(vd <= 64 ? 64 : 128), 0, st, part_o, part_ml,
-                         (bf16*)out, out_ld, nsplit, nseq, H, vd, out_scale);
+                         (bf16*)out, out_ld, nsplit, nseq, H, vd, out_scale, ex);
     return hipGetLastError();
   }
   const size_t bytes = ((size_t)d + 4 * 64 + 8 + 4 * (size_t)vd) * sizeof(float);
   if (dt == 0 && d % 8 == 0 && vd % 2 == 0 && vd <= 256 && v_ld % 2 == 0 && (reinterpret_cast<uintptr_t>(v_cache) & 3) == 0) {
     hipLaunchKernelGGL(sink_attn_decode_vec_kernel, dim3(H, nseq), dim3(256), bytes, st, (const bf16*)q,
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,
-                       ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld);
+                       ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld, ex);
     return hipGetLastError();
   }
   DT_DISPATCH(dt, hipLaunchKernelGGL(sink_attn_decode_kernel<T>, dim3(H, nseq), dim3(256), bytes, st, (const T*)q,
                                      (const T*)k_cache, (const T*)v_cache, (T*)out, out_ld, block_tables, bt_stride,
-                                     ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld);)
+                                     ctx_len, sinks, H, G, d, vd, BS, scale, out_scale, nblocks, v_ld, ex);)
   return hipGetLastError();
 }
 
@@ -1368,7 +1417,7 @@ GRAG_API hipError_t grag_window_decode_mfma(const void* q, const void* k_cache, 
     hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV, 1>), mgrid, dim3(256), mb, st, (const bf16*)q,          \
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
                        ctx_len, bias, H, G, d, vd, BS, scale, 1.f, nblocks, 1, 0, (float*)nullptr, (float*)nullptr,  \
-                       window, (const bf16*)gate, gate_ld, vd);                                                      \
+                       window, (const bf16*)gate, gate_ld, vd, AttnExtra{nullptr, nullptr, 0, 0});                   \
   }
   if (d <= 64 && vd <= 64) SW_MFMA(4, 4)
   else SW_MFMA(8, 8)

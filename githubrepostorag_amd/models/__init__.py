@@ -18,6 +18,10 @@ def build_decoder(cfg, **kw):
         from .namudra import NamudraModel
 
         return NamudraModel(cfg, **kw)
+    if cfg.arch == "leripel":
+        from .leripel import LeripelModel
+
+        return LeripelModel(cfg, **kw)
     from .qwen2 import Qwen2Model
 
     return Qwen2Model(cfg, **kw)

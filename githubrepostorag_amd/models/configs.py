@@ -138,14 +138,63 @@ class LatentAttnSpec:
 
 
 @dataclass(frozen=True)
+class ChunkAttnSpec:
+    """Softmax attention inside aligned blocks of ``chunk`` positions (0: plain causal), GQA, partial rotary on
+    adjacent pairs, a temperature per head, a sigmoid output gate per head."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    chunk: int
+    rot_dims: int
+    rot_base: float
+
+
+@dataclass(frozen=True)
+class SSMSpec:
+    """State-space mixer: ``heads`` heads of ``vdim`` channels with an [state, vdim] fp32 state each, B / C shared by
+    the heads of each of ``groups`` groups, a causal convolution of ``taps`` taps in front, a gated RMS norm in
+    ``norm_groups`` parts behind."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    norm_groups: int
+    taps: int
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.heads * self.vdim + 2 * self.groups * self.state
+
+
+@dataclass(frozen=True)
+class MoESpec:
+    """Mixture of SiLU-gated experts: ``top`` of ``experts`` per token, chosen among the ``keep`` best of ``groups``
+    equal groups of neighbours, weighted by their softmax scores; a shared expert of ``shared_ff`` (0: none) with a
+    sigmoid gate per token."""
+    kind: str  # "moe"
+    ff: int
+    experts: int
+    top: int
+    groups: int
+    keep: int
+    shared_ff: int
+
+
+@dataclass(frozen=True)
 class MixerSpec:
-    kind: str  # "parallel" | "mingru" | "retention" | "attention" | "latent_attention"
+    kind: str  # "parallel" | "mingru" | "retention" | "attention" | "latent_attention" | "mamba2"
     left: SinkAttnSpec | None = None
     right: DecayAttnSpec | None = None
     left_scale: float = 1.0
     right_scale: float = 1.0
     width: int = 0  # mingru state width
-    spec: RetentionSpec | WindowAttnSpec | LatentAttnSpec | None = None  # the single-mixer kinds
+    spec: RetentionSpec | WindowAttnSpec | LatentAttnSpec | ChunkAttnSpec | SSMSpec | None = None  # single-mixer kinds
 
 
 @dataclass(frozen=True)
@@ -158,7 +207,7 @@ class GLUSpec:
 @dataclass(frozen=True)
 class HybridLayerSpec:
     mixer: MixerSpec
-    mlp: GLUSpec | None
+    mlp: GLUSpec | MoESpec | None
 
 
 @dataclass(frozen=True)
@@ -197,6 +246,22 @@ class HybridConfig:
 
     def param_count(self) -> int:
         H = self.hidden_size
+        if self.arch == "leripel":
+            n = 2 * self.vocab_size * H + H + (2 * H * H if self.loop_stop > self.loop_start else 0)
+            for L in self.layers:
+                m, a = L.mixer.kind, L.mixer.spec
+                n += H
+                if m == "retention":
+                    n += H * a.heads * (2 * a.dim + 2 * a.vdim) + a.heads * a.vdim * H
+                elif m == "attention":
+                    n += H * (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim) + a.heads) + a.heads + a.heads * a.vdim * H
+                else:
+                    n += H * (2 * a.inner + 2 * a.groups * a.state + a.heads) + a.conv_channels * (a.taps + 1)
+                    n += 3 * a.heads + a.inner + a.inner * H
+                if L.mlp is not None:
+                    f = L.mlp
+                    n += f.experts * (3 * H * f.ff + H) + (3 * H * f.shared_ff + H if f.shared_ff else 0)
+            return n
         if self.arch == "namudra":
             S = self.streams
             n = 2 * self.vocab_size * H + H
@@ -366,6 +431,97 @@ def namudra_config(name: str, vocab: int, width: int, pattern: str, *, heads: in
                         streams=streams)
 
 
+def leripel_config_from_dict(d: dict, name: str = "leripel") -> HybridConfig:
+    """The Leripel design's config.json: a layer list of "retention" / "attention" / "mamba2" mixers, each beside an
+    optional mixture-of-experts feed-forward that reads the same normed input; an optional loop whose every pass
+    re-enters through a projection of [x; embedding].  Every size and constant is read from it."""
+    layers = []
+    for e in d["layers"]:
+        kind, m = e["type"], e["mixer"]
+        if kind == "retention":
+            a = RetentionSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), tuple(float(x) for x in m["decay"]), 0, 1.0)
+            if len(a.decay) != a.heads:
+                raise ValueError(f"bad retention sizes {m}")
+        elif kind == "attention":
+            rot = m.get("rot") or {"dims": 0, "base": 1.0}
+            mask = m.get("mask") or {"size": 0}
+            a = ChunkAttnSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]),
+                              int(m.get("vdim", m["dim"])), float(m["scale"]), int(mask.get("size", 0)),
+                              int(rot["dims"]), float(rot.get("base", 1.0)))
+            if a.heads % a.kv_heads or a.rot_dims % 2 or a.rot_dims > a.dim or a.chunk < 0:
+                raise ValueError(f"bad attention sizes {m}")
+        elif kind == "mamba2":
+            a = SSMSpec(int(m["heads"]), int(m["vdim"]), int(m["state"]), int(m.get("groups", 1)),
+                        int(m.get("norm_groups", 1)), int(m["conv"]))
+            if a.heads % a.groups or a.inner % a.norm_groups or a.taps < 1:
+                raise ValueError(f"bad state-space sizes {m}")
+        else:
+            raise ValueError(f"unknown mixer type {kind!r}")
+        f = e.get("mlp")
+        if f is None:
+            mlp = None
+        elif f.get("kind", "moe") == "moe":
+            r = f["router"]
+            g = r.get("groups") or {"count": 1, "keep": 1}
+            sh = f.get("shared")
+            mlp = MoESpec("moe", int(f["expert"]["ff"]), int(r["experts"]), int(r["top"]), int(g["count"]),
+                          int(g["keep"]), int(sh["ff"]) if sh else 0)
+            if mlp.experts % mlp.groups or not 1 <= mlp.keep <= mlp.groups or not 1 <= mlp.top <= mlp.experts:
+                raise ValueError(f"bad router sizes {r}")
+        else:
+            raise ValueError(f"unknown feed-forward kind {f.get('kind')!r}")
+        layers.append(HybridLayerSpec(MixerSpec(kind, spec=a), mlp))
+    loop = d.get("loop") or {}
+    return HybridConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]), tuple(layers),
+                        int(loop.get("start", 0)), int(loop.get("stop", 0)), int(loop.get("times", 1)), arch="leripel")
+
+
+def leripel_config_to_dict(cfg: HybridConfig) -> dict:
+    """Back to the config.json form (checkpoint export, tests)."""
+    layers = []
+    for L in cfg.layers:
+        a, kind = L.mixer.spec, L.mixer.kind
+        if kind == "retention":
+            m = {"heads": a.heads, "dim": a.dim, "vdim": a.vdim, "decay": list(a.decay)}
+        elif kind == "attention":
+            m = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale,
+                 "mask": {"size": a.chunk}, "rot": {"dims": a.rot_dims, "base": a.rot_base}}
+        else:
+            m = {"heads": a.heads, "vdim": a.vdim, "state": a.state, "groups": a.groups,
+                 "norm_groups": a.norm_groups, "conv": a.taps}
+        f = L.mlp
+        mlp = None if f is None else {
+            "kind": "moe", "expert": {"ff": f.ff},
+            "router": {"experts": f.experts, "top": f.top, "groups": {"count": f.groups, "keep": f.keep}},
+            "shared": {"ff": f.shared_ff} if f.shared_ff else None}
+        layers.append({"type": kind, "mixer": m, "mlp": mlp})
+    return {"architecture": "Leripel", "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+            "norm": {"eps": cfg.norm_eps}, "layers": layers,
+            "loop": {"start": cfg.loop_start, "stop": cfg.loop_stop, "times": cfg.loop_times}}
+
+
+def leripel_config(name: str, vocab: int, width: int, pattern: str, *, heads: int, kv_heads: int, dim: int,
+                   chunk: int = 2048, rot_dims: int | None = None, ret_heads: int | None = None,
+                   ret_dim: int | None = None, ret_vdim: int | None = None, ssm_heads: int | None = None,
+                   ssm_vdim: int = 64, ssm_state: int = 128, ssm_groups: int = 1, ssm_norm_groups: int = 1,
+                   taps: int = 4, experts: int = 16, top: int = 4, groups=(4, 2), ff: int = 1024,
+                   shared_ff: int = 0, loop=(0, 0, 1), eps: float = 1e-5, moe: bool = True) -> HybridConfig:
+    """A regular Leripel stack for benches and plumbing tests.  ``pattern``: one letter per layer, r = retention,
+    a = block-local attention, m = state-space mixer; every layer carries the same mixture of experts."""
+    rh, rdm, rvd = ret_heads or heads, ret_dim or dim, ret_vdim or dim
+    decay = tuple(1.0 - 2.0 ** (-4.0 - 6.0 * i / max(1, rh - 1)) for i in range(rh))
+    sh = ssm_heads or max(1, width // ssm_vdim)
+    mlp = MoESpec("moe", ff, experts, top, groups[0], groups[1], shared_ff) if moe else None
+    kinds = {
+        "r": MixerSpec("retention", spec=RetentionSpec(rh, rdm, rvd, decay, 0, 1.0)),
+        "a": MixerSpec("attention", spec=ChunkAttnSpec(heads, kv_heads, dim, dim, dim ** -0.5, chunk,
+                                                       dim // 2 if rot_dims is None else rot_dims, 1e4)),
+        "m": MixerSpec("mamba2", spec=SSMSpec(sh, ssm_vdim, ssm_state, ssm_groups, ssm_norm_groups, taps)),
+    }
+    return HybridConfig(name, vocab, width, eps, tuple(HybridLayerSpec(kinds[c], mlp) for c in pattern), *loop,
+                        arch="leripel")
+
+
 def zofesun_config(name: str, vocab: int, width: int, n_layers: int, *, heads: int, kv_heads: int, dim: int,
                    vdim: int, lin_heads: int, lin_dim: int, lin_vdim: int, ff: int, mingru_every: int = 0,
                    rot_dims: int | None = None, rot_base: float = 10000.0, loop=(0, 0, 1), limit: float = 7.0,
@@ -397,6 +553,18 @@ HYBRIDS = {
                                  window=1024, kv_rank=192, q_rank=384, rot_dim=64, ret_ff=True),
     "namudra-7b": namudra_config("namudra-7b", 32768, 3584, "rala", heads=28, kv_heads=4, dim=128, ff=18944,
                                  window=1024, kv_rank=192, q_rank=768, rot_dim=64, ret_ff=True),
+    # Leripel: a plumbing-test size and two bench sizes with the layer shapes of a 1.5B / 7B decoder (the routed
+    # experts' active width top * ff plus the shared expert equals the dense decoders' feed-forward width)
+    "leripel-tiny": leripel_config("leripel-tiny", 320, 96, "rama", heads=4, kv_heads=2, dim=16, chunk=9, rot_dims=8,
+                                   ret_heads=3, ret_dim=8, ret_vdim=24, ssm_heads=6, ssm_vdim=8, ssm_state=12,
+                                   ssm_groups=2, ssm_norm_groups=3, experts=6, top=2, groups=(3, 2), ff=40,
+                                   shared_ff=56, loop=(1, 3, 2)),
+    "leripel-1b": leripel_config("leripel-1b", 32768, 1536, "ramarama", heads=12, kv_heads=2, dim=128, chunk=1024,
+                                 ssm_vdim=64, ssm_state=128, experts=16, top=4, groups=(4, 2), ff=1792,
+                                 shared_ff=1792),
+    "leripel-7b": leripel_config("leripel-7b", 32768, 3584, "rama", heads=28, kv_heads=4, dim=128, chunk=1024,
+                                 ssm_vdim=64, ssm_state=128, experts=16, top=4, groups=(4, 2), ff=3840,
+                                 shared_ff=3584),
 }
 
 
@@ -409,6 +577,8 @@ def config_from_dir(path) -> DecoderConfig | HybridConfig:
         return hybrid_config_from_dict(d, Path(path).name or "zofesun")
     if arch == "namudra":
         return namudra_config_from_dict(d, Path(path).name or "namudra")
+    if arch == "leripel":
+        return leripel_config_from_dict(d, Path(path).name or "leripel")
     mt = str(d.get("model_type", "")).lower()
     if mt == "gpt2":
         return DecoderConfig(Path(path).name, d["vocab_size"], d["n_embd"], d.get("n_inner") or 4 * d["n_embd"],

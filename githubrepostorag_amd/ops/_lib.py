@@ -81,9 +81,9 @@ _SIGS = {
     "grag_err_alloc": [P],
     "grag_embed_f32": [P, P, P, I, I, I, I, P],
     "grag_dyt_residual": [P, F, P, P, P, P, P, F, P, P, P, I, I, I, P],
-    "grag_rope_vnorm_store": [P, I, I, I, I, P, P, I, P, P, P, P, I, I, I, I, I, I, I, ctypes.c_long, F, I, P],
-    "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P],
-    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, I, I, P, P, I, P],
+    "grag_rope_vnorm_store": [P, I, I, I, I, P, P, I, P, P, P, P, I, I, I, I, I, I, I, ctypes.c_long, F, I, I, P],
+    "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P, P, I, I, P],
+    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, I, I, P, P, I, P, P, I, I, P],
     "grag_decay_attn_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, P, P, I, I, F, P],
     "grag_decay_attn_chunk": [],
     "grag_mingru_chunk": [],
@@ -99,6 +99,16 @@ _SIGS = {
     "grag_rmsnorm_rows": [P, I, P, P, I, I, F, I, P],
     "grag_window_decode_mfma": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, I, P, I, P],
     "grag_attn_decode_xcd": [I],
+    "grag_conv_max_taps": [],
+    "grag_causal_conv": [P, I, I, I, I, P, P, P, P, P, P, P, I, I, I, I, P],
+    "grag_ssm_chunk": [],
+    "grag_ssm_scan": [P, I, I, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, P, I, P],
+    "grag_moe_max_rows": [],
+    "grag_moe_max_top": [],
+    "grag_moe_route": [P, I, P, I, I, I, I, I, I, P, P, P, I, I, P],
+    "grag_moe_align": [P, I, I, P, P, P],
+    "grag_moe_gemm": [P, I, P, P, P, I, I, I, I, I, P, I, I, I, P],
+    "grag_residual_rmsnorm": [P, F, P, P, P, P, P, I, P, F, P, P, I, I, I, I, P],
 }
 
 
@@ -165,7 +175,7 @@ def call(name: str, *args) -> None:
 
 
 # ---------------------------------------------------------------- device index guard (csrc/kernels/common.h)
-ERR_UNITS = ("norm", "elementwise", "attention", "gemm_tile", "gemm_stream", "seqmix", "gatedmix")
+ERR_UNITS = ("norm", "elementwise", "attention", "gemm_tile", "gemm_stream", "seqmix", "gatedmix", "ssm", "moe")
 ERR_CODES = {1 << 0: "embed_gather: token id >= vocab", 1 << 1: "qkv_rope_kvstore: KV slot id >= cache slots",
              1 << 2: "qkv_rope_kvstore: position >= RoPE table rows",
              1 << 3: "prefill attention: block-table entry >= KV blocks",

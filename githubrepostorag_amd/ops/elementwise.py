@@ -159,10 +159,12 @@ def rope_table(max_pos: int, rot_dims: int, base: float, device=None) -> torch.T
 
 def rope_vnorm_store(proj: torch.Tensor, qoff: int, koff: int, voff: int, positions: torch.Tensor,
                      table: torch.Tensor, slot_mapping: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                     H: int, G: int, d: int, vd: int, rot_dims: int, eps: float) -> torch.Tensor:
+                     H: int, G: int, d: int, vd: int, rot_dims: int, eps: float, interleaved: bool = False,
+                     vnorm: bool = True) -> torch.Tensor:
     """From a fused projection ``proj`` [T, ld] (q heads at column qoff, k at koff, v at voff): rotate the first
-    ``rot_dims`` dims of every q / k head (dim i paired with i + rot_dims/2), divide every v head by its root
-    mean square (fp32), store k / v into the paged caches k_cache [blocks, G, BS, d] / v_cache [blocks, G, BS, vd]
+    ``rot_dims`` dims of every q / k head (dim i paired with i + rot_dims/2; ``interleaved``: dim 2i with 2i + 1,
+    pair i turned by the table's angle i), divide every v head by its root mean square (fp32; ``vnorm`` False: the
+    values as they are), store k / v into the paged caches k_cache [blocks, G, BS, d] / v_cache [blocks, G, BS, vd]
     at ``slot_mapping`` (-1: not stored) and return q [T, H, d]."""
     T = proj.shape[0]
     BS = k_cache.shape[2]
@@ -176,10 +178,16 @@ def rope_vnorm_store(proj: torch.Tensor, qoff: int, koff: int, voff: int, positi
             cs = table[positions.long()]
             c, s = cs[:, None, :h2], cs[:, None, h2:]
             for t in (q, k):
+                if interleaved:
+                    a, b = t[..., 0:rot_dims:2].clone(), t[..., 1:rot_dims:2].clone()
+                    t[..., 0:rot_dims:2] = a * c - b * s
+                    t[..., 1:rot_dims:2] = b * c + a * s
+                    continue
                 a, b = t[..., :h2].clone(), t[..., h2:rot_dims].clone()
                 t[..., :h2] = a * c - b * s
                 t[..., h2:rot_dims] = b * c + a * s
-        v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        if vnorm:
+            v = v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps)
         ok = slot_mapping >= 0
         sl = slot_mapping[ok].long()
         k_cache[sl // BS, :, sl % BS] = k[ok].to(k_cache.dtype)
@@ -188,8 +196,9 @@ def rope_vnorm_store(proj: torch.Tensor, qoff: int, koff: int, voff: int, positi
     assert proj.stride(1) == 1 and k_cache.dtype == proj.dtype and v_cache.dtype == proj.dtype
     q = torch.empty(T, H, d, dtype=proj.dtype, device=proj.device)
     call("grag_rope_vnorm_store", ptr(proj), proj.stride(0), qoff, koff, voff, ptr(positions), ptr(table),
-         table.shape[0], ptr(slot_mapping), ptr(q), ptr(k_cache), ptr(v_cache), T, H, G, d, vd, rot_dims, BS,
-         k_cache.shape[0] * BS, float(eps), 0 if proj.dtype == torch.bfloat16 else 1)
+         0 if table is None else table.shape[0], ptr(slot_mapping), ptr(q), ptr(k_cache), ptr(v_cache), T, H, G, d, vd, rot_dims, BS,
+         k_cache.shape[0] * BS, float(eps), 0 if proj.dtype == torch.bfloat16 else 1,
+         (1 if interleaved else 0) | (0 if vnorm else 2))
     return q
 
 

@@ -225,3 +225,43 @@ def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
     call("grag_rmsnorm_rows", ptr(x), x.stride(0), ptr(w), ptr(out), T, N, float(eps),
          0 if x.dtype == torch.bfloat16 else 1)
     return out
+
+
+# ---------------------------------------------------------------------------------------------- parallel-block boundary
+def residual_rmsnorm(x: torch.Tensor, a: torch.Tensor | None = None, b: torch.Tensor | None = None,
+                     bcoef: torch.Tensor | None = None, e: torch.Tensor | None = None,
+                     ecoef: torch.Tensor | None = None, w: torch.Tensor | None = None, eps: float = 1e-6,
+                     out_dtype=torch.bfloat16, keep: bool = True, raw: torch.Tensor | None = None):
+    """One pass over the fp32 residual ``x`` [T, H] (updated in place) at the boundary of a layer whose sublayers
+    read the same input: x <- x + (a + bcoef_t b + sum_k ecoef[t, k] e[t, k]) with every addend optional
+    (``a``, ``b`` [T, H]; ``bcoef`` [T] fp32, None: 1; ``e`` [T, K, H] with ``ecoef`` [T, K] fp32), all summed in
+    fp32; ``keep`` False: x is replaced by the sum instead.  ``raw`` [T, H] (a column slice of a wider buffer is
+    fine): receives x in ``out_dtype``.  With ``w`` [H] fp32 returns x / sqrt(mean(x^2) + eps) * w in ``out_dtype``."""
+    assert x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
+    T, H = x.shape
+    K = 0 if e is None else e.shape[1]
+    if not _on_gpu(x):
+        y = torch.zeros_like(x)
+        if a is not None:
+            y += a.float()
+        f = torch.zeros_like(x)
+        if b is not None:
+            f += b.float() * (1.0 if bcoef is None else bcoef.float()[:, None])
+        if e is not None:
+            f += (e.float() * ecoef.float()[:, :, None]).sum(1)
+        y += f
+        x.copy_(x + y if keep else y)
+        if raw is not None:
+            raw.copy_(x.to(raw.dtype))
+        return None if w is None else (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+    for t in (a, b):
+        assert t is None or (t.dtype == out_dtype and t.is_contiguous() and t.shape == (T, H))
+    assert e is None or (e.dtype == out_dtype and e.is_contiguous() and e.shape == (T, K, H)
+                         and ecoef.dtype == torch.float32 and ecoef.is_contiguous() and ecoef.shape == (T, K))
+    assert bcoef is None or (bcoef.dtype == torch.float32 and bcoef.numel() == T)
+    assert raw is None or (raw.dtype == out_dtype and raw.stride(1) == 1 and raw.shape == (T, H))
+    out = torch.empty(T, H, dtype=out_dtype, device=x.device) if w is not None else None
+    call("grag_residual_rmsnorm", ptr(x), 1.0 if keep else 0.0, ptr(a), ptr(b), ptr(bcoef), ptr(e), ptr(ecoef), K,
+         ptr(w), float(eps), ptr(out), ptr(raw), 0 if raw is None else raw.stride(0), T, H,
+         0 if out_dtype == torch.bfloat16 else 1)
+    return out

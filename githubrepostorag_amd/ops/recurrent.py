@@ -99,23 +99,25 @@ def _decay_attention_cpu(x, qoff, koff, voff, decay, state, m, H, d, vd, out, ac
 
 
 def gated_rmsnorm(x: torch.Tensor, w: torch.Tensor | None, proj: torch.Tensor, goff: int, eps: float,
-                  out: torch.Tensor, out_scale: float = 1.0, groups: int = 1, gate: str = "sigmoid") -> torch.Tensor:
+                  out: torch.Tensor, out_scale: float = 1.0, groups: int = 1, gate: str = "sigmoid",
+                  gate_first: bool = False) -> torch.Tensor:
     """out = out_scale * x / rms(x) * w * gate(g): x [T, N] fp32 normalised over each of ``groups`` equal column
     groups (1: the whole row; the head count: per head), ``w`` [N] optional, g read from columns goff.. of the
-    fused projection, gate "sigmoid" or "silu"; ``out`` [T, N] may be a column slice of a wider buffer."""
+    fused projection, gate "sigmoid" or "silu"; ``out`` [T, N] may be a column slice of a wider buffer.
+    ``gate_first``: the gate comes before the norm, out = out_scale * u / rms(u) * w with u = x * gate(g)."""
     T, N = x.shape
     if gate not in ("sigmoid", "silu") or N % groups:
         raise ValueError("gate is 'sigmoid' or 'silu', and the groups divide the row")
     if not x.is_cuda:
         g = proj[:, goff:goff + N].float()
         g = torch.sigmoid(g) if gate == "sigmoid" else torch.nn.functional.silu(g)
-        xg = x.view(T, groups, N // groups)
+        xg = (x * g if gate_first else x).view(T, groups, N // groups)
         y = (xg / torch.sqrt(xg.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, N)
-        out.copy_(y * (1.0 if w is None else w.float()) * g * out_scale)
+        out.copy_(y * (1.0 if w is None else w.float()) * (1.0 if gate_first else g) * out_scale)
         return out
     assert x.is_contiguous() and out.stride(1) == 1 and out.dtype == proj.dtype
     call("grag_gated_rmsnorm", ptr(x), ptr(w), ptr(proj), proj.stride(0), goff, ptr(out), out.stride(0), T, N,
-         float(eps), float(out_scale), _dt(proj), groups, 1 if gate == "silu" else 0)
+         float(eps), float(out_scale), _dt(proj), groups, (1 if gate == "silu" else 0) | (2 if gate_first else 0))
     return out
 
 
@@ -154,4 +156,96 @@ def _mingru_cpu(x, zoff, xoff, goff, bz, bx, state, m, W, out):
         for t in range(a, b):
             S = (1.0 - z[t]) * S + z[t] * c[t]
             out[t] = (S * g[t]).to(out.dtype)
+        state[sl[s]] = S
+
+
+# ---------------------------------------------------------------------------------------------- state-space mixer
+def causal_conv(proj: torch.Tensor, coff: int, w: torch.Tensor, b: torch.Tensor | None, cstate: torch.Tensor,
+                meta: AttnMetadata) -> torch.Tensor:
+    """Causal depthwise convolution + SiLU over columns coff .. coff + C of the fused projection ``proj`` [T, ld]:
+    out[t, c] = silu(b[c] + sum_j w[c, j] in[t - (taps - 1) + j, c]) with ``w`` [C, taps] fp32 (the last tap is the
+    current token's).  Inputs before a portion come from ``cstate`` [slots, taps - 1, C] (the sequence's last
+    taps - 1 inputs, oldest first; zeros for a sequence that starts at position 0), which is brought up to date
+    after the step.  Returns [T, C] in proj's dtype."""
+    T = proj.shape[0]
+    C, taps = w.shape
+    out = torch.empty(T, C, dtype=proj.dtype, device=proj.device)
+    for m, r0, r1 in _parts(meta):
+        if r1 <= r0:
+            continue
+        if not proj.is_cuda:
+            _causal_conv_cpu(proj[r0:r1], coff, w, b, cstate, m, out[r0:r1])
+            continue
+        assert proj.stride(1) == 1 and cstate.dtype == proj.dtype and cstate.is_contiguous() and w.is_contiguous()
+        assert w.dtype == torch.float32 and cstate.shape[1:] == (taps - 1, C) and taps <= lib().grag_conv_max_taps()
+        call("grag_causal_conv", ptr(proj[r0:r1]), proj.stride(0), coff, C, taps, ptr(w), ptr(b), ptr(cstate),
+             ptr(m.state_slots), ptr(m.q_start), ptr(m.ctx_len), ptr(out[r0:r1]), m.num_seqs, m.max_q_len,
+             cstate.shape[0], _dt(proj))
+    return out
+
+
+def _causal_conv_cpu(x, coff, w, b, cstate, m, out):
+    C, taps = w.shape
+    qs, cl, sl = m.q_start.tolist(), m.ctx_len.tolist(), m.state_slots.tolist()
+    for s in range(m.num_seqs):
+        a, e = qs[s], qs[s + 1]
+        if e <= a:
+            continue
+        past = torch.zeros(taps - 1, C) if cl[s] - (e - a) == 0 else cstate[sl[s]].float()
+        full = torch.cat([past, x[a:e, coff:coff + C].float()], 0)
+        acc = torch.zeros(e - a, C) if b is None else b.float().expand(e - a, C).clone()
+        for j in range(taps):
+            acc += w[:, j].float() * full[j:j + (e - a)]
+        out[a:e] = torch.nn.functional.silu(acc).to(out.dtype)
+        if taps > 1:
+            cstate[sl[s]] = full[-(taps - 1):].to(cstate.dtype)
+
+
+def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dtoff: int, dt_bias: torch.Tensor, a_log: torch.Tensor,
+             skip: torch.Tensor, state: torch.Tensor, meta: AttnMetadata, H: int, G: int, N: int, P: int) -> torch.Tensor:
+    """Selective state-space scan.  ``xbc`` [T, H*P + 2*G*N] (the convolution's output): x heads | B groups | C groups;
+    the step sizes' raw values are columns dtoff .. dtoff + H of ``proj``.  Per head h (group h // (H / G)), in fp32:
+    dt = softplus(raw + dt_bias[h]), S_t = exp(-exp(a_log[h]) dt) S_(t-1) + dt B_t x_t^T (state [slots, H, N, P]),
+    y_t = S_t^T C_t + skip[h] x_t.  Returns y [T, H*P] fp32."""
+    T = xbc.shape[0]
+    out = torch.empty(T, H * P, dtype=torch.float32, device=xbc.device)
+    C = xbc.shape[1]
+    assert C == H * P + 2 * G * N
+    for m, r0, r1 in _parts(meta):
+        if r1 <= r0:
+            continue
+        if not xbc.is_cuda:
+            _ssm_scan_cpu(xbc[r0:r1].float(), proj[r0:r1, dtoff:dtoff + H].float(), dt_bias, a_log, skip, state, m, H, G,
+                          N, P, out[r0:r1])
+            continue
+        assert xbc.is_contiguous() and proj.stride(1) == 1 and state.dtype == torch.float32 and state.is_contiguous()
+        assert xbc.dtype == proj.dtype and state.shape[1:] == (H, N, P)
+        chunk = lib().grag_ssm_chunk()
+        ws = wa = None
+        if m.max_q_len > chunk:
+            nch = m.num_seqs * -(-m.max_q_len // chunk)
+            ws = torch.empty(nch * H * N * P, dtype=torch.float32, device=xbc.device)
+            wa = torch.empty(nch * H, dtype=torch.float32, device=xbc.device)
+        call("grag_ssm_scan", ptr(xbc[r0:r1]), C, H * P, H * P + G * N, ptr(proj[r0:r1]), proj.stride(0), dtoff,
+             ptr(dt_bias), ptr(a_log), ptr(skip), ptr(state), ptr(m.state_slots), ptr(m.q_start), ptr(m.ctx_len),
+             ptr(out[r0:r1]), m.num_seqs, H, G, N, P, state.shape[0], _dt(xbc), ptr(ws), ptr(wa), m.max_q_len)
+    return out
+
+
+def _ssm_scan_cpu(xbc, dtraw, dt_bias, a_log, skip, state, m, H, G, N, P, out):
+    qs, cl, sl = m.q_start.tolist(), m.ctx_len.tolist(), m.state_slots.tolist()
+    dt = torch.nn.functional.softplus(dtraw + dt_bias.float(), threshold=20.0)
+    decay = torch.exp(-torch.exp(a_log.float()) * dt)
+    R = H // G
+    for s in range(m.num_seqs):
+        a, e = qs[s], qs[s + 1]
+        if e <= a:
+            continue
+        S = torch.zeros(H, N, P) if cl[s] - (e - a) == 0 else state[sl[s]].clone()
+        x = xbc[a:e, :H * P].view(-1, H, P)
+        B = xbc[a:e, H * P:H * P + G * N].view(-1, G, N).repeat_interleave(R, dim=1)
+        Cm = xbc[a:e, H * P + G * N:].view(-1, G, N).repeat_interleave(R, dim=1)
+        for t in range(e - a):
+            S = decay[a + t, :, None, None] * S + (dt[a + t, :, None] * B[t])[:, :, None] * x[t][:, None, :]
+            out[a + t] = (torch.einsum("hnp,hn->hp", S, Cm[t]) + skip.float()[:, None] * x[t]).reshape(-1)
         state[sl[s]] = S
