@@ -1,0 +1,304 @@
+"""Scenarios that compare the engine serving a Leripel model (kernels, paged cache, state slots, scheduler) with
+the plain float64 oracle of leripel_oracle.py.  Every scenario takes the device: the CPU tier runs the ops' host
+paths, the GPU tier the HIP kernels, through the same engine code."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+import leripel_oracle as O
+
+
+def build(cfg_dict, sd, device, dtype=torch.float32, slots=4, pool_tokens=512, block_size=16, graphs=False,
+          max_batched=4096, mixed=False, window=1):
+    from githubrepostorag_amd.engine.llm_engine import EngineConfig, LLMEngine
+    from githubrepostorag_amd.models import build_decoder
+    from githubrepostorag_amd.models.configs import leripel_config_from_dict
+
+    model = build_decoder(leripel_config_from_dict(cfg_dict), device=device, dtype=dtype, state_dict=sd)
+    eng = LLMEngine(model, None, EngineConfig(max_num_seqs=slots, max_model_len=max(pool_tokens, 64),
+                                              block_size=block_size, num_blocks=pool_tokens // block_size + 1,
+                                              use_cuda_graph=graphs, max_num_batched_tokens=max_batched,
+                                              mixed_batches=mixed, decode_window=window))
+    return model, eng
+
+
+def tokens(cfg, n, seed):
+    g = torch.Generator().manual_seed(9000 + seed)
+    return torch.randint(0, cfg["vocab"], (n,), generator=g).tolist()
+
+
+def rel_err(got, want):
+    """Mean-free RMS difference over the vocabulary, relative to the logits' own spread (per row, the worst)."""
+    got = torch.as_tensor(np.asarray(got), dtype=torch.float64)
+    want = torch.as_tensor(np.asarray(want), dtype=torch.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdim=True)
+    return float((d.pow(2).mean(-1).sqrt() / want.std(-1)).max())
+
+
+def feed_in_portions(eng, rid, toks, cuts, end=True):
+    """Feed ``toks`` as portions of the sizes in ``cuts`` (cycled), asking for every place; -> logits [T, vocab]."""
+    out, a, i = [], 0, 0
+    while a < len(toks):
+        n = min(cuts[i % len(cuts)], len(toks) - a)
+        last = a + n == len(toks)
+        out.append(eng.feed([(rid, toks[a:a + n], list(range(n)))], [rid] if last and end else []))
+        a += n
+        i += 1
+    return np.concatenate(out, 0)
+
+
+def case_whole_and_layers(device, tol, dtype=torch.float32, **cfg_kw):
+    cfg = O.make_config(**cfg_kw)
+    sd = O.make_weights(cfg, seed=3)
+    toks = tokens(cfg, 33, 0)
+    want, taps = O.logits_and_taps(cfg, sd, toks)
+    model, eng = build(cfg, sd, device, dtype)
+    assert rel_err(feed_in_portions(eng, "a", toks, [len(toks)]), want) < tol
+    # the residual after every layer run, through the model's own step (one sequence, fresh cache / state)
+    from githubrepostorag_amd.ops.attention import AttnMetadata
+
+    T, bs = len(toks), 16
+    nb = -(-T // bs)
+    i32 = dict(dtype=torch.int32, device=model.device)
+    meta = AttnMetadata(q_start=torch.tensor([0, T], **i32), ctx_len=torch.tensor([T], **i32),
+                        block_tables=(torch.arange(nb, **i32) + 1).view(1, nb), slot_mapping=torch.arange(T, **i32) + bs,
+                        max_q_len=T, num_seqs=1, num_tokens=T, state_slots=torch.tensor([1], **i32))
+    mine = []
+    model.forward(torch.tensor(toks, **i32), torch.arange(T, **i32), meta, model.allocate_kv_cache(nb + 1, bs),
+                  state=model.allocate_state(2), taps=mine)
+    assert len(mine) == taps.shape[0]
+    for r, (a, b) in enumerate(zip(mine, taps)):
+        err = float((a.double().cpu() - b).abs().max() / b.abs().max())
+        assert err < tol, (r, err)
+
+
+def case_single_mixer(device, tol, kind, dtype=torch.float32, mlp=False, **kw):
+    """One layer of one mixer (with or without the experts beside it): the mechanism alone between embedding and
+    head; whole, token by token, and in portions."""
+    cfg = O.make_config(kinds=(kind,), loop=(0, 0, 1), no_mlp=() if mlp else (0,), **kw)
+    sd = O.make_weights(cfg, seed=21)
+    toks = tokens(cfg, 41, 5)
+    want = O.forward(cfg, sd, toks)
+    _, eng = build(cfg, sd, device, dtype)
+    assert rel_err(feed_in_portions(eng, "w", toks, [41]), want) < tol
+    assert rel_err(feed_in_portions(eng, "d", toks, [1]), want) < tol
+    assert rel_err(feed_in_portions(eng, "c", toks, [6, 2, 19]), want) < tol
+
+
+def case_prefill_vs_decode(device, tol, dtype=torch.float32, n=58, **cfg_kw):
+    cfg = O.make_config(**cfg_kw)
+    sd = O.make_weights(cfg, seed=5)
+    toks = tokens(cfg, n, 1)
+    want = O.forward(cfg, sd, toks)
+    _, eng = build(cfg, sd, device, dtype)
+    assert rel_err(feed_in_portions(eng, "p", toks, [n]), want) < tol
+    assert rel_err(feed_in_portions(eng, "d", toks, [1]), want) < tol           # every token on the decode path
+    assert rel_err(feed_in_portions(eng, "pd", toks, [n - 20] + [1] * 20), want) < tol  # blocks end among decoded tokens
+
+
+def case_portions(device, tol, dtype=torch.float32):
+    """Portions cut inside pages (16), attention blocks (7), the convolution's reach (3) and scan chunks (64), down
+    to two tokens."""
+    cfg = O.make_config(kinds=("mamba2", "attention", "retention", "mamba2"), loop=(0, 2, 3), no_mlp=(1,))
+    sd = O.make_weights(cfg, seed=7)
+    toks = tokens(cfg, 139, 2)
+    want = O.forward(cfg, sd, toks)
+    _, eng = build(cfg, sd, device, dtype)
+    for k, cuts in enumerate(([2], [3, 2, 17, 1, 16, 31], [16], [15, 1, 1, 33], [64, 2], [65, 63, 11], [130, 9], [1, 2])):
+        assert rel_err(feed_in_portions(eng, f"c{k}", toks, cuts), want) < tol, cuts
+
+
+def case_batches(device, tol, dtype=torch.float32):
+    """Unequal requests in one batch -- portions beside single tokens, requests that sit out steps and end at
+    different times -- give each request the logits it gets alone."""
+    cfg = O.make_config()
+    sd = O.make_weights(cfg, seed=9)
+    lens = {"a": 45, "b": 9, "c": 31, "d": 18}
+    toks = {k: tokens(cfg, n, 10 + i) for i, (k, n) in enumerate(lens.items())}
+    want = {k: O.forward(cfg, sd, t) for k, t in toks.items()}
+    _, eng = build(cfg, sd, device, dtype, pool_tokens=192)
+    plan = [  # (request, tokens) per step
+        [("a", 20), ("b", 2)],
+        [("a", 1), ("b", 1), ("c", 17)],
+        [("a", 1), ("c", 1), ("d", 16)],
+        [("b", 6), ("a", 3), ("d", 1), ("c", 13)],
+        [("a", 20), ("d", 1)],
+    ]
+    cur = {k: 0 for k in toks}
+    got = {k: [] for k in toks}
+    for step in plan:
+        entries, end = [], []
+        for k, n in step:
+            entries.append((k, toks[k][cur[k]:cur[k] + n], list(range(n))))
+            cur[k] += n
+            if cur[k] == lens[k]:
+                end.append(k)
+        out = eng.feed(entries, end)
+        o = 0
+        for k, n in step:
+            got[k].append(out[o:o + n])
+            o += n
+    for k in toks:
+        assert cur[k] == lens[k]
+        assert rel_err(np.concatenate(got[k], 0), want[k]) < tol, k
+    assert eng.kv.num_free == eng.kv.num_blocks - 1 and len(eng.sched.free_slots) == 4
+
+
+def case_reuse(device, tol, dtype=torch.float32):
+    """Pages and state slots that were freed are used again: with one slot and a pool of two requests' worth,
+    later requests land on the earlier ones' pages, convolution inputs and states and still match their oracle."""
+    cfg = O.make_config(loop=(0, 0, 1))
+    sd = O.make_weights(cfg, seed=11)
+    _, eng = build(cfg, sd, device, dtype, slots=1, pool_tokens=64)
+    for i, n in enumerate((50, 7, 33, 64, 1)):
+        toks = tokens(cfg, n, 20 + i)
+        want = O.forward(cfg, sd, toks)
+        cuts = [[n], [3, 1], [32, 1], [60, 2, 1, 1], [1]][i]
+        assert rel_err(feed_in_portions(eng, f"r{i}", toks, cuts), want) < tol, i
+        assert eng.kv.num_free == eng.kv.num_blocks - 1
+    # a request that stops mid-way leaves nothing behind either
+    eng.feed([("x", tokens(cfg, 40, 30), [])], [])
+    eng.feed([], ["x"])
+    toks = tokens(cfg, 21, 31)
+    assert rel_err(feed_in_portions(eng, "y", toks, [20, 1]), O.forward(cfg, sd, toks)) < tol
+
+
+def case_long_decode(device, tol, dtype=torch.float32):
+    cfg = O.make_config(kinds=("retention", "mamba2", "attention"), loop=(0, 2, 2), ret_heads=3,
+                        decay=[0.2, 0.9, 0.9995], chunk=33)
+    sd = O.make_weights(cfg, seed=13)
+    toks = tokens(cfg, 150, 3)
+    want = O.forward(cfg, sd, toks)
+    _, eng = build(cfg, sd, device, dtype)
+    assert rel_err(feed_in_portions(eng, "l", toks, [6] + [1] * 144), want) < tol
+
+
+def case_other_sizes(device, tol, dtype=torch.float32):
+    """Sizes where things the usual configs make equal differ, or are 1."""
+    variants = [
+        # one kv head, whole-head rotary, value size above the key size, blocks of one position; one retention head
+        # with dim > vdim; one expert group, every expert chosen; no shared expert
+        dict(width=40, vocab=33, kinds=("retention", "attention"), loop=(0, 2, 2), heads=3, kv_heads=1, dim=10, vdim=24,
+             rot_dims=10, rot_base=7.0, scale=1.0, chunk=1, ret_heads=1, ret_dim=10, ret_vdim=6, decay=[0.97],
+             experts=3, top=3, groups=(1, 1), shared_ff=None),
+        # heads == kv heads, no rotary, a block longer than the prompt; one state-space head, one group, one norm part,
+        # a convolution of one tap; top 1; as many groups as experts
+        dict(width=48, vocab=50, kinds=("attention", "mamba2"), loop=(0, 0, 1), heads=2, kv_heads=2, dim=72, vdim=72,
+             rot_dims=0, scale=0.1, chunk=500, ssm_heads=1, ssm_vdim=20, ssm_state=5, ssm_groups=1, ssm_norm_groups=1,
+             taps=1, experts=4, top=1, groups=(4, 2), ff=8, shared_ff=8),
+        # decay 1 (nothing forgotten) and a fast one; value size above 64; the loop is the whole stack and runs three
+        # times; a state wider than its heads; two taps; no feed-forward in the second layer; keep == count
+        dict(width=56, vocab=64, kinds=("mamba2", "retention"), loop=(0, 2, 3), no_mlp=(1,), ret_heads=2, ret_dim=20,
+             ret_vdim=70, decay=[1.0, 0.5], ssm_heads=6, ssm_vdim=4, ssm_state=40, ssm_groups=3, ssm_norm_groups=2,
+             taps=2, experts=8, top=5, groups=(2, 2)),
+        # a loop that runs once, blocks of two, five taps
+        dict(loop=(1, 2, 1), chunk=2, taps=5),
+        # no loop at all (and so no re-entry projection)
+        dict(loop=(0, 0, 1), kinds=("attention", "mamba2", "retention")),
+    ]
+    for i, kw in enumerate(variants):
+        cfg = O.make_config(**kw)
+        sd = O.make_weights(cfg, seed=40 + i)
+        toks = tokens(cfg, 29, 40 + i)
+        want = O.forward(cfg, sd, toks)
+        _, eng = build(cfg, sd, device, dtype)
+        assert rel_err(feed_in_portions(eng, "w", toks, [29]), want) < tol, i
+        assert rel_err(feed_in_portions(eng, "c", toks, [5, 1, 2]), want) < tol, i
+
+
+def case_first_tokens(device, tol, dtype=torch.float32):
+    """Position 0 alone (one key, a state and a convolution that start from zeros in a used slot), then 1, 2."""
+    cfg = O.make_config()
+    sd = O.make_weights(cfg, seed=17)
+    _, eng = build(cfg, sd, device, dtype, slots=1)
+    eng.feed([("warm", tokens(cfg, 30, 50), [])], ["warm"])  # leave a state and pages behind
+    for n in (1, 2, 3, 5):
+        toks = tokens(cfg, n, 60 + n)
+        want = O.forward(cfg, sd, toks)
+        assert rel_err(feed_in_portions(eng, f"f{n}", toks, [1]), want) < tol
+        assert rel_err(feed_in_portions(eng, f"g{n}", toks, [n]), want) < tol
+
+
+def case_sharp_far_keys(device, tol, dtype=torch.float32):
+    """A softmax scale large enough that every query picks out single keys of its block, many of them far back and
+    across page borders: a key read from the wrong place changes the logits outright.  300 tokens in blocks of
+    150, the last 40 decoded one by one, portions cut off the page grid."""
+    cfg = O.make_config(kinds=("attention",), loop=(0, 1, 2), no_mlp=(0,), scale=6.0, chunk=150, kv_heads=1)
+    sd = O.make_weights(cfg, seed=29)
+    toks = tokens(cfg, 300, 6)
+    want = O.forward(cfg, sd, toks)
+    _, eng = build(cfg, sd, device, dtype)
+    assert rel_err(feed_in_portions(eng, "s", toks, [300]), want) < tol
+    assert rel_err(feed_in_portions(eng, "t", toks, [97, 130, 33] + [1] * 40), want) < tol
+
+
+def case_block_edges(device, tol, dtype=torch.float32, bs=16):
+    """The attention op alone on crafted keys: key j is 30 e_j, so a query e_p scores 30 on position p and 0
+    elsewhere, and the softmax weight of an asked-for visible key is ~1.  Head 0 asks for the first key of the
+    query's own block (just inside), head 1 for the last key of the block before (just outside: its weight must
+    be spread over the visible keys instead, none of which carries the marker value), head 2 for the query's own
+    position.  In a prompt's portion that follows cached context and for a decoded token; blocks that end on,
+    before and after page borders, pages out of order; temperatures and gates per head."""
+    from githubrepostorag_amd.ops.attention import AttnMetadata, sink_attention
+
+    dev = torch.device(device)
+    H, G, ctx = 3, 1, 75
+    d, vd = 80, 16
+    for chunk in (1, 5, bs, bs + 1, 2 * bs - 1, 40, 0):
+        nb = -(-ctx // bs)
+        g = torch.Generator().manual_seed(chunk)
+        perm = (torch.randperm(nb, generator=g) + 1).to(torch.int32)
+        kc = torch.zeros(nb + 1, G, bs, d, dtype=dtype, device=dev)
+        vc = torch.zeros(nb + 1, G, bs, vd, dtype=dtype, device=dev)
+        V = torch.zeros(ctx, vd)
+        V[:, 0] = torch.arange(ctx) + 1.0  # the value names its position
+        for j in range(ctx):
+            kc[perm[j // bs], 0, j % bs, j] = 30.0
+            vc[perm[j // bs], 0, j % bs] = V[j].to(dtype)
+        temp = torch.tensor([1.0, 1.0, 0.5], device=dev)
+        for qlen in (33, 9, 1):  # (33 queries in bf16: the matrix-core kernel)
+            q = torch.zeros(qlen, H, d)
+            gate = torch.randn(qlen, H, generator=g)
+            for n, p in enumerate(range(ctx - qlen, ctx)):
+                lo = p - p % chunk if chunk else 0
+                q[n, 0, lo] = 1.0
+                if lo > 0:
+                    q[n, 1, lo - 1] = 1.0
+                q[n, 2, p] = 2.0  # (half the temperature: the same score)
+            i32 = dict(dtype=torch.int32, device=dev)
+            meta = AttnMetadata(q_start=torch.tensor([0, qlen], **i32), ctx_len=torch.tensor([ctx], **i32),
+                                block_tables=perm.view(1, nb).to(dev), slot_mapping=torch.zeros(qlen, **i32),
+                                max_q_len=qlen, num_seqs=1, num_tokens=qlen, is_decode=qlen == 1)
+            got = sink_attention(q.to(dtype).to(dev), kc, vc, meta, 1.0, None, head_scale=temp,
+                                 head_gate=gate.to(dtype).to(dev), chunk=chunk).float().cpu().view(qlen, H, vd)
+            sg = torch.sigmoid(gate.to(dtype).float())
+            for n, p in enumerate(range(ctx - qlen, ctx)):
+                lo = p - p % chunk if chunk else 0
+                assert abs(float(got[n, 0, 0]) / float(sg[n, 0]) - (lo + 1.0)) < tol * ctx, (chunk, qlen, p, "inside")
+                assert abs(float(got[n, 2, 0]) / float(sg[n, 2]) - (p + 1.0)) < tol * ctx, (chunk, qlen, p, "self")
+                if lo > 0:  # the key just outside gets nothing: head 1 sees a flat average of its block's values
+                    want = float(V[lo:p + 1, 0].mean())
+                    assert abs(float(got[n, 1, 0]) / float(sg[n, 1]) - want) < tol * ctx, (chunk, qlen, p, "outside")
+
+
+def case_generate(device, dtype=torch.float32, graphs=False, mixed=False, window=1, max_batched=4096, tol=2e-3,
+                  **cfg_kw):
+    """Greedy generation through LLMEngine.generate (scheduler, chunked prefill, sampler, decode steps): every
+    generated token is the oracle's arg-max given the tokens before it (up to a near-tie)."""
+    from githubrepostorag_amd.engine.sequence import SamplingParams
+
+    cfg = O.make_config(**cfg_kw)
+    sd = O.make_weights(cfg, seed=19)
+    _, eng = build(cfg, sd, device, dtype, slots=3, pool_tokens=256, graphs=graphs, mixed=mixed, window=window,
+                   max_batched=max_batched)
+    prompts = [tokens(cfg, n, 70 + i) for i, n in enumerate((5, 23, 11, 2))]  # 4 prompts on 3 slots: one waits
+    outs = eng.generate(prompts, SamplingParams(max_tokens=10, temperature=0.0, ignore_eos=True))
+    for p, c in zip(prompts, outs):
+        assert len(c.token_ids) == 10
+        logits = O.forward(cfg, sd, p + c.token_ids[:-1])
+        for j, t in enumerate(c.token_ids):
+            row = logits[len(p) - 1 + j]
+            assert float(row.max() - row[t]) < tol * float(row.std()), (len(p), j)
+    assert eng.kv.num_free == eng.kv.num_blocks - 1
