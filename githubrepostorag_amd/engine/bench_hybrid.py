@@ -1,9 +1,10 @@
-"""``bench.py --hybrid [zofesun|namudra]``: prefill and decode throughput of a hybrid decoder beside the decoders of
+"""``bench.py --hybrid [zofesun|namudra|leripel]``: prefill and decode throughput of a hybrid decoder beside the decoders of
 equal size that the engine already serves (same width, heads, head size, FFN width, layer count, vocabulary; random
 weights, synthetic token ids), all through LLMEngine.generate, and a per-kernel table: each new kernel and the
 like kernel of the closest model as a fraction of the roofline of what bounds it (HBM bytes or matrix / vector
 flops).  Zofesun stands beside Qwen2; Namudra beside Zofesun (the closest: fp32 residual, decay scan, sink
-attention kernels) and Qwen2."""
+attention kernels) and Qwen2; Leripel beside Namudra (the closest: fp32 residual, retention scan, the same attention
+kernel family, a layer list that is data) and Qwen2."""
 from __future__ import annotations
 
 import json
@@ -283,6 +284,171 @@ def _namudra_kernel_table(dev, H=28, G=4, D=128, W=3584, T=2048, B=64, ctx=2048,
     return rows
 
 
+def _leripel_models(name, dev):
+    """Leripel at a bench size: per four layers retention, block-local attention (blocks of 1024), the state-space
+    mixer, block-local attention; every layer beside a mixture of 16 experts (4 per token) plus a shared expert whose
+    active width equals the dense decoders' feed-forward; beside the Namudra and Qwen2 stacks."""
+    from ..models.configs import leripel_config
+    from ..models.leripel import LeripelModel
+
+    W, H, G, D, ff, nl, _ = SIZES[name]
+    per = (ff // 5) // 64 * 64
+    lc = leripel_config(f"leripel-{name}", VOCAB, W, ("rama" * nl)[:nl], heads=H, kv_heads=G, dim=D, chunk=1024,
+                        ssm_vdim=64, ssm_state=128, experts=16, top=4, groups=(4, 2), ff=per, shared_ff=ff - 4 * per)
+    mk_n, _, mk_q = _namudra_models(name, dev)
+    return (lambda: LeripelModel(lc, device=dev, seed=1)), mk_n, mk_q
+
+
+def _leripel_kernel_table(dev, H=28, G=4, D=128, W=3584, ff=18944, T=2048, B=64, ctx=2048, bs=16, chunk=1024, E=16,
+                          top=4, P=64, N=128):
+    """[(kernel, seconds, bound, fraction of roofline)] for Leripel's kernels and the like kernels of Namudra."""
+    from ..ops.attention import AttnMetadata, sigmoid_window_attention, sink_attention
+    from ..ops.elementwise import rope_table, rope_vnorm_store
+    from ..ops.linear import linear
+    from ..ops.moe import moe_experts, moe_route
+    from ..ops.norm import hyper_mix, residual_rmsnorm
+    from ..ops.recurrent import causal_conv, decay_attention, gated_rmsnorm, ssm_scan
+
+    bf = torch.bfloat16
+    i32 = dict(dtype=torch.int32, device=dev)
+    rows = []
+
+    def add(name, sec, flops=0.0, bytes_=0.0, peak=MFMA_BF16):
+        t_c, t_m = flops / peak, bytes_ / HBM_BPS
+        rows.append({"kernel": name, "us": round(sec * 1e6, 1), "bound": "flops" if t_c >= t_m else "bytes",
+                     "roofline_fraction": round(max(t_c, t_m) / sec, 4)})
+
+    nb = T // bs
+    meta = AttnMetadata(q_start=torch.tensor([0, T], **i32), ctx_len=torch.tensor([T], **i32),
+                        block_tables=(torch.arange(nb, **i32) + 1).view(1, nb), slot_mapping=torch.arange(T, **i32) + bs,
+                        max_q_len=T, num_seqs=1, num_tokens=T, state_slots=torch.tensor([0], **i32))
+    nbd = ctx // bs
+    dmeta = AttnMetadata(q_start=torch.arange(B + 1, **i32), ctx_len=torch.full((B,), ctx, **i32),
+                         block_tables=(torch.arange(B * nbd, **i32) + 1).view(B, nbd), slot_mapping=None, max_q_len=1,
+                         num_seqs=B, num_tokens=B, is_decode=True, state_slots=torch.arange(B, **i32))
+    # ---- attention: blocks of `chunk` positions, temperatures, head gates | sliding window of the same length
+    kc = torch.randn(nb + 1, G, bs, D, device=dev).to(bf)
+    vc = torch.randn(nb + 1, G, bs, D, device=dev).to(bf)
+    q = torch.randn(T, H, D, device=dev).to(bf)
+    temp, pb = torch.ones(H, device=dev), torch.zeros(H, device=dev)
+    hg = torch.randn(T, H, device=dev).to(bf)
+    gate = torch.randn(T, H * D, device=dev).to(bf)
+    pairs_c = (T // chunk) * chunk * (chunk + 1) / 2
+    pairs_w = T * (T + 1) / 2 - (T - chunk) * (T - chunk + 1) / 2
+    add(f"block-local attention prefill (blocks of {chunk})",
+        _timed(lambda: sink_attention(q, kc, vc, meta, 0.09, None, head_scale=temp, head_gate=hg, chunk=chunk)),
+        flops=4.0 * pairs_c * H * D)
+    add("namudra sigmoid_window_prefill (window 1024)",
+        _timed(lambda: sigmoid_window_attention(q, kc, vc, meta, 0.09, pb, chunk, gate=gate)), flops=4.0 * pairs_w * H * D)
+    kd = torch.randn(B * nbd + 1, G, bs, D, device=dev).to(bf)
+    vd_ = torch.randn(B * nbd + 1, G, bs, D, device=dev).to(bf)
+    qd = torch.randn(B, H, D, device=dev).to(bf)
+    hgd = torch.randn(B, H, device=dev).to(bf)
+    gd = torch.randn(B, H * D, device=dev).to(bf)
+    dmeta.ctx_len = torch.full((B,), ctx, **i32)  # the last token closes a block: a full block of keys is read
+    add(f"block-local attention decode ({chunk} keys)",
+        _timed(lambda: sink_attention(qd, kd, vd_, dmeta, 0.09, None, head_scale=temp, head_gate=hgd, chunk=chunk)),
+        bytes_=2.0 * B * chunk * G * D * 2)
+    add("namudra sigmoid_window_decode (window 1024)",
+        _timed(lambda: sigmoid_window_attention(qd, kd, vd_, dmeta, 0.09, pb, chunk, gate=gd)), bytes_=2.0 * B * chunk * G * D * 2)
+    # ---- rotary + K/V store
+    proj = torch.randn(T, (H + 2 * G) * D + 32, device=dev).to(bf)
+    pos = torch.arange(T, **i32)
+    tab, tabh = rope_table(T, D, 1e4, dev), rope_table(T, D // 2, 1e4, dev)
+    by = T * (H + 2 * G) * D * 2 * 2.0
+    add("rope store, adjacent pairs, half the head", _timed(lambda: rope_vnorm_store(
+        proj, 0, H * D, (H + G) * D, pos, tabh, meta.slot_mapping, kc, vc, H, G, D, D, D // 2, 1e-5, interleaved=True,
+        vnorm=False)), bytes_=by)
+    add("zofesun rope_vnorm_store", _timed(lambda: rope_vnorm_store(proj, 0, H * D, (H + G) * D, pos, tab, meta.slot_mapping,
+                                                                    kc, vc, H, G, D, D, D, 1e-5)), bytes_=by)
+    # ---- layer boundary: mixer + shared + `top` weighted experts into one fp32 residual | two fp32 streams
+    x = torch.randn(T, W, device=dev)
+    a, b = torch.randn(T, W, device=dev).to(bf), torch.randn(T, W, device=dev).to(bf)
+    e = torch.randn(T, top, W, device=dev).to(bf)
+    ec, bc, w32 = torch.rand(T, top, device=dev), torch.rand(T, device=dev), torch.ones(W, device=dev)
+    add(f"residual_rmsnorm (mixer + shared + {top} experts)", _timed(lambda: residual_rmsnorm(x, a, b, bc, e, ec, w32, 1e-5)),
+        bytes_=T * W * (8 + 2.0 * (2 + top) + 2))
+    xs = torch.randn(2, T, W, device=dev)
+    mix, oc, ic = torch.eye(2, device=dev), torch.ones(2, device=dev), torch.ones(2, device=dev) / 2
+    add("namudra hyper_mix (2 fp32 streams)", _timed(lambda: hyper_mix(xs, a, mix, oc, ic, w32, 1e-6)), bytes_=T * W * (2 + 16.0 + 2))
+    # ---- state-space mixer | retention scan
+    Hs = W // P
+    inner, ch = Hs * P, Hs * P + 2 * N
+    ld = 2 * inner + 2 * N + Hs
+    pj = (torch.randn(T, ld, device=dev) * 0.5).to(bf)
+    cw, cb = torch.randn(ch, 4, device=dev) * 0.5, torch.zeros(ch, device=dev)
+    cst = torch.zeros(B + 1, 3, ch, device=dev, dtype=bf)
+    sst = torch.zeros(B + 1, Hs, N, P, device=dev)
+    dtb, alog, dsk = torch.zeros(Hs, device=dev), torch.zeros(Hs, device=dev), torch.ones(Hs, device=dev)
+    add("causal_conv prefill (4 taps)", _timed(lambda: causal_conv(pj, inner, cw, cb, cst, meta)), bytes_=T * ch * 2 * 2.0)
+    xbc = causal_conv(pj, inner, cw, cb, cst, meta)
+    add("ssm_scan prefill", _timed(lambda: ssm_scan(xbc, pj, inner + ch, dtb, alog, dsk, sst, meta, Hs, 1, N, P), 3, 1),
+        flops=4.0 * T * Hs * N * P, bytes_=T * ch * 2.0, peak=VALU_F32)
+    pr = torch.randn(T, 4 * H * D, device=dev).to(bf)
+    dec = torch.full((H,), 0.99, device=dev)
+    St = torch.zeros(B + 1, H, D, D, device=dev)
+    add("retention scan prefill (no rotary)", _timed(lambda: decay_attention(pr, 0, H * D, 2 * H * D, dec, St, meta, H, D, D, act=False,
+                                                                             k_scale=D ** -0.5), 3, 1),
+        flops=4.0 * T * H * D * D, bytes_=T * 3 * H * D * 2.0, peak=VALU_F32)
+    pjd = (torch.randn(B, ld, device=dev) * 0.5).to(bf)
+    add("causal_conv decode", _timed(lambda: causal_conv(pjd, inner, cw, cb, cst, dmeta)), bytes_=B * ch * 2 * (2 + 2 * 3.0))
+    xbd = causal_conv(pjd, inner, cw, cb, cst, dmeta)
+    add("ssm_scan decode", _timed(lambda: ssm_scan(xbd, pjd, inner + ch, dtb, alog, dsk, sst, dmeta, Hs, 1, N, P)),
+        bytes_=2.0 * B * Hs * N * P * 4)
+    prd = torch.randn(B, 4 * H * D, device=dev).to(bf)
+    add("retention scan decode", _timed(lambda: decay_attention(prd, 0, H * D, 2 * H * D, dec, St, dmeta, H, D, D, act=False,
+                                                               k_scale=D ** -0.5)), bytes_=2.0 * B * H * D * D * 4)
+    o = torch.randn(T, inner, device=dev)
+    out = torch.empty(T, inner, device=dev, dtype=bf)
+    add("gated_rmsnorm, gate first, whole row", _timed(lambda: gated_rmsnorm(o, w32[:inner].contiguous(), pj, 0, 1e-5, out, gate="silu",
+                                                                             gate_first=True)), bytes_=T * inner * (4 + 2 + 2.0))
+    o2 = torch.randn(T, H * D, device=dev)
+    out2 = torch.empty(T, H * D, device=dev, dtype=bf)
+    add("namudra gated_rmsnorm per head", _timed(lambda: gated_rmsnorm(o2, None, pr, 3 * H * D, 1e-6, out2, groups=H, gate="silu")),
+        bytes_=T * H * D * (4 + 2 + 2.0))
+    # ---- experts: router, grouped GEMMs | dense GEMMs of the same active width through the engine's linear()
+    F = (ff // 5) // 64 * 64
+    h = torch.randn(T, W, device=dev).to(bf)
+    wr = torch.randn(E + 1, W, device=dev) * 0.05
+    add("moe_route (16 experts + gate row)", _timed(lambda: moe_route(h, wr, E, top, 4, 2)), flops=2.0 * T * (E + 1) * W,
+        bytes_=T * W * 2.0, peak=VALU_F32)
+    ids, _, _ = moe_route(h, wr, E, top, 4, 2)
+    wgu = (torch.randn(E, 2 * F, W, device=dev) * 0.02).to(bf)
+    wd = (torch.randn(E, W, F, device=dev) * 0.02).to(bf)
+    add(f"moe experts prefill ({T} x {top} rows, align + 2 grouped GEMMs)", _timed(lambda: moe_experts(h, ids, wgu, wd)),
+        flops=6.0 * T * top * F * W)
+    wgd, wdd = (torch.randn(2 * top * F, W, device=dev) * 0.02).to(bf), (torch.randn(W, top * F, device=dev) * 0.02).to(bf)
+    hh = torch.randn(T, top * F, device=dev).to(bf)
+    add("dense gate|up + down GEMMs of the same active width (linear)",
+        _timed(lambda: (linear(h, wgd), linear(hh, wdd))), flops=6.0 * T * top * F * W)
+    hd = torch.randn(B, W, device=dev).to(bf)
+    idd, _, _ = moe_route(hd, wr, E, top, 4, 2)
+    add(f"moe experts decode ({B} x {top} rows)", _timed(lambda: moe_experts(hd, idd, wgu, wd)), bytes_=3.0 * E * F * W * 2)
+    hhd = torch.randn(B, top * F, device=dev).to(bf)
+    add("dense gate|up + down GEMMs, decode rows (linear)", _timed(lambda: (linear(hd, wgd), linear(hhd, wdd))),
+        bytes_=3.0 * top * F * W * 2)
+    return rows
+
+
+def run_leripel(args) -> dict:
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    sizes = {}
+    for name in SIZES:
+        makers = dict(zip(("leripel", "namudra", "qwen2"), _leripel_models(name, dev)))
+        cell = {}
+        for batch, plen, glen in ((8, 2048, 64), (64, 1024, 64)):
+            key = f"B{batch}_P{plen}_G{glen}"
+            cell[key] = {k: _engine_numbers(mk, dev, batch, plen, glen) for k, mk in makers.items()}
+            print(json.dumps({"size": name, "shape": key, **cell[key]}), flush=True)
+        sizes[name] = cell
+    kernels = _leripel_kernel_table(dev)
+    for r in kernels:
+        print(json.dumps(r), flush=True)
+    return {"metric": "leripel_vs_namudra_vs_qwen2_tokens_per_s", "unit": "tokens/s", "dtype": "bf16",
+            "data": "synthetic", "sizes": sizes, "kernels": kernels}
+
+
 def run_namudra(args) -> dict:
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
@@ -305,6 +471,8 @@ def run_namudra(args) -> dict:
 def run(args) -> dict:
     if getattr(args, "hybrid", None) == "namudra":
         return run_namudra(args)
+    if getattr(args, "hybrid", None) == "leripel":
+        return run_leripel(args)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     sizes = {}
