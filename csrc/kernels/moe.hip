@@ -22,7 +22,8 @@ template <> __device__ __forceinline__ void stm<float>(float* p, float v) { *p =
 
 // ------------------------------------------------------------------------------------------------ router
 constexpr int RT_TOK = 16;    // tokens per workgroup
-constexpr int RT_KC = 32;     // columns of h / the router matrix staged per step
+constexpr int RT_KC = 128;    // columns of h / the router matrix staged per step
+constexpr int RT_LD = RT_KC + 4;  // LDS row stride (floats): 16-byte rows, banks spread over the rows
 constexpr int RT_MAXR = 256;  // logit rows (experts + the shared gate's row) at most
 constexpr int RT_MAXTOP = 16;
 
@@ -34,10 +35,11 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ wr, int W, int E, int R, int top,
                  int ngroups, int keep, int* __restrict__ ids, float* __restrict__ wts, float* __restrict__ sgate,
-                 int T_) {
-  __shared__ float hs[RT_TOK][RT_KC + 1];
-  __shared__ float ws[RT_MAXR][RT_KC + 1];
-  __shared__ float lg[RT_TOK][RT_MAXR + 1];
+                 int T_, int vec) {
+  extern __shared__ __attribute__((aligned(16))) float rsm[];
+  float* hs = rsm;                   // [RT_TOK][RT_LD]
+  float* ws = hs + RT_TOK * RT_LD;   // [R][RT_LD]
+  float* lgs = ws + (size_t)R * RT_LD;  // [RT_TOK][R + 1]
   const int tok = threadIdx.x & 15, part = threadIdx.x >> 4;
   const int t0 = blockIdx.x * RT_TOK;
   float acc[RT_MAXR / 16];
@@ -45,32 +47,76 @@ moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ wr, 
   for (int j = 0; j < RT_MAXR / 16; ++j) acc[j] = 0.f;
   for (int k0 = 0; k0 < W; k0 += RT_KC) {
     __syncthreads();
+    if (vec) {
+      // 16-byte loads, all of the step's loads in flight before the first LDS store (W a multiple of 8: a vector
+      // never straddles the row's end).  h: thread t -> token t / 16, columns 8 (t % 16) .. + 7; wr: float4 c of row r
+      // for idx = r * 32 + c
+      const int tt = threadIdx.x >> 4, kv = (threadIdx.x & 15) * 8;
+      float hv[8];
+      const bool hok = t0 + tt < T_ && k0 + kv < W;
+      if (sizeof(T) == 2) {
+        const bf16x8_t v = hok ? *reinterpret_cast<const bf16x8_t*>(h + (size_t)(t0 + tt) * ld + k0 + kv)
+                               : bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) hv[i] = bits2f(v[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) hv[i] = hok ? ldm(h + (size_t)(t0 + tt) * ld + k0 + kv + i) : 0.f;
+      }
+      const int nvec = R * (RT_KC / 4);
+      for (int base = 0; base < nvec; base += 256 * 4) {
+        f32x4_t wv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int idx = base + threadIdx.x + 256 * u;
+          const int r = idx / (RT_KC / 4), c = idx - r * (RT_KC / 4);
+          wv[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          if (idx < nvec && k0 + 4 * c < W) wv[u] = *reinterpret_cast<const f32x4_t*>(wr + (size_t)r * W + k0 + 4 * c);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int idx = base + threadIdx.x + 256 * u;
+          const int r = idx / (RT_KC / 4), c = idx - r * (RT_KC / 4);
+          if (idx < nvec) *reinterpret_cast<f32x4_t*>(ws + r * RT_LD + 4 * c) = wv[u];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) hs[tt * RT_LD + kv + i] = hv[i];
+    } else
     for (int idx = threadIdx.x; idx < RT_TOK * RT_KC; idx += 256) {
       const int tt = idx / RT_KC, k = idx - tt * RT_KC;
-      hs[tt][k] = (t0 + tt < T_ && k0 + k < W) ? ldm(h + (size_t)(t0 + tt) * ld + k0 + k) : 0.f;
+      hs[tt * RT_LD + k] = (t0 + tt < T_ && k0 + k < W) ? ldm(h + (size_t)(t0 + tt) * ld + k0 + k) : 0.f;
     }
-    for (int idx = threadIdx.x; idx < R * RT_KC; idx += 256) {
+    for (int idx = threadIdx.x; !vec && idx < R * RT_KC; idx += 256) {
       const int r = idx / RT_KC, k = idx - r * RT_KC;
-      ws[r][k] = k0 + k < W ? wr[(size_t)r * W + k0 + k] : 0.f;
+      ws[r * RT_LD + k] = k0 + k < W ? wr[(size_t)r * W + k0 + k] : 0.f;
     }
     __syncthreads();
+    const f32x4_t* h4 = reinterpret_cast<const f32x4_t*>(hs + tok * RT_LD);
 #pragma unroll
     for (int j = 0; j < RT_MAXR / 16; ++j) {
       const int r = part + 16 * j;
       if (r < R) {
+        const f32x4_t* w4 = reinterpret_cast<const f32x4_t*>(ws + r * RT_LD);
         float a = acc[j];
-#pragma unroll
-        for (int k = 0; k < RT_KC; ++k) a = fmaf(hs[tok][k], ws[r][k], a);
+#pragma unroll 8
+        for (int k = 0; k < RT_KC / 4; ++k) {  // (k ascending: one fixed summation order per logit)
+          const f32x4_t hv = h4[k], wv = w4[k];
+          a = fmaf(hv[0], wv[0], a);
+          a = fmaf(hv[1], wv[1], a);
+          a = fmaf(hv[2], wv[2], a);
+          a = fmaf(hv[3], wv[3], a);
+        }
         acc[j] = a;
       }
     }
   }
 #pragma unroll
   for (int j = 0; j < RT_MAXR / 16; ++j)
-    if (part + 16 * j < R) lg[tok][part + 16 * j] = acc[j];
+    if (part + 16 * j < R) lgs[tok * (R + 1) + part + 16 * j] = acc[j];
   __syncthreads();
   if (threadIdx.x >= RT_TOK || t0 + threadIdx.x >= T_) return;
-  float* z = lg[threadIdx.x];
+  float* z = lgs + threadIdx.x * (R + 1);
   const int t = t0 + threadIdx.x;
   if (R > E && sgate != nullptr) sgate[t] = 1.f / (1.f + expf(-z[E]));
   float mx = -INFINITY;
@@ -328,6 +374,118 @@ moe_gemm_mfma_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict
   }
 }
 
+// Large tiles for prompt-sized row counts (bf16): 128 rows x 128 columns per workgroup, 4 waves of 64 x 64 (wave w: rows
+// 64 (w / 2), columns 64 (w % 2)), v_mfma_f32_16x16x32_bf16 (operand lane: row / column lane % 16, k = 8 (lane / 16)
+// .. + 7), K steps of 64 (one 128-byte line per row) staged through LDS with the next step's global loads in flight
+// during the products.
+template <int GATED>
+__global__ void __launch_bounds__(256, 2)
+moe_gemm_big_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, const int* __restrict__ offs,
+                    const int* __restrict__ order, int E, int top, int N, int K, bf16* __restrict__ out, int ldo) {
+  constexpr int TM = 128, TN = 128, TK = 64, KS = TK + 8, NB = GATED ? 2 : 1;
+  __shared__ __attribute__((aligned(16))) short As[TM][KS];
+  __shared__ __attribute__((aligned(16))) short Bs[NB][TN][KS];
+  __shared__ int rows[TM];
+  int e = 0, tile = blockIdx.y, r0 = -1, rend = 0;
+  for (; e < E; ++e) {
+    const int b = offs[e], n = offs[e + 1] - b, nt = (n + TM - 1) / TM;
+    if (tile < nt) {
+      r0 = b + tile * TM;
+      rend = b + n;
+      break;
+    }
+    tile -= nt;
+  }
+  if (r0 < 0) return;
+  const int n0 = blockIdx.x * TN;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int ql = lane & 15, quad = lane >> 4;
+  const int wr = (wid >> 1) * 64, wc = (wid & 1) * 64;
+  if (threadIdx.x < TM) {
+    const int r = r0 + threadIdx.x;
+    rows[threadIdx.x] = r < rend ? (GATED ? order[r] / top : r) : -1;
+  }
+  __syncthreads();
+  const size_t wrows = GATED ? (size_t)2 * N : (size_t)N;
+  const bf16* we = w + (size_t)e * wrows * K;
+  // staging: thread t owns rows t / 8 + 32 u (u < 4) of every tile, 16-byte vector (t % 8) of the K step
+  constexpr int NU = 4;
+  const int sr = threadIdx.x >> 3, sv = (threadIdx.x & 7) * 8;
+  const bf16* ap[NU];
+  const bf16* bp[NB][NU];
+  bool aok[NU], bok[NU];
+#pragma unroll
+  for (int u = 0; u < NU; ++u) {
+    const int src = rows[sr + 32 * u];
+    aok[u] = src >= 0;
+    ap[u] = a + (size_t)(aok[u] ? src : 0) * lda + sv;
+    bok[u] = n0 + sr + 32 * u < N;
+#pragma unroll
+    for (int g = 0; g < NB; ++g) bp[g][u] = we + ((size_t)g * N + (bok[u] ? n0 + sr + 32 * u : 0)) * K + sv;
+  }
+  const bf16x8_t zero = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8_t av[NU], bv[NB][NU];
+  auto fetch = [&](int k0) {
+    const bool kok = k0 + sv < K;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      av[u] = (aok[u] && kok) ? *reinterpret_cast<const bf16x8_t*>(ap[u] + k0) : zero;
+#pragma unroll
+      for (int g = 0; g < NB; ++g) bv[g][u] = (bok[u] && kok) ? *reinterpret_cast<const bf16x8_t*>(bp[g][u] + k0) : zero;
+    }
+  };
+  f32x4_t acc[NB][4][4];
+#pragma unroll
+  for (int g = 0; g < NB; ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[g][i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += TK) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      *reinterpret_cast<bf16x8_t*>(&As[sr + 32 * u][sv]) = av[u];
+#pragma unroll
+      for (int g = 0; g < NB; ++g) *reinterpret_cast<bf16x8_t*>(&Bs[g][sr + 32 * u][sv]) = bv[g][u];
+    }
+    __syncthreads();
+    if (k0 + TK < K) fetch(k0 + TK);
+#pragma unroll
+    for (int ks = 0; ks < TK / 32; ++ks) {
+      bf16x8_t af[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8_t*>(&As[wr + 16 * i + ql][ks * 32 + quad * 8]);
+#pragma unroll
+      for (int g = 0; g < NB; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bf16x8_t bf = *reinterpret_cast<const bf16x8_t*>(&Bs[g][wc + 16 * j + ql][ks * 32 + quad * 8]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[g][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf, acc[g][i][j], 0, 0, 0);
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int r = r0 + wr + 16 * i + 4 * quad + c;
+      if (r >= rend) continue;
+      const size_t orow = GATED ? (size_t)r : (size_t)order[r];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + wc + 16 * j + ql;
+        if (n >= N) continue;
+        float v = acc[0][i][j][c];
+        if (GATED) v = v / (1.f + expf(-v)) * acc[NB - 1][i][j][c];
+        out[orow * ldo + n] = (bf16)v;
+      }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ residual boundary
 // x [T][H] fp32, in place: x <- keep x + (a + bcoef_t b + sum_k ecoef_(t,k) e_(t,k)), every addend optional
 // (a, b [T][H]; e [T * K][H], ecoef [T * K]; bcoef [T], null: 1).  Then, each optional: raw [T][raw_ld] <- x in the
@@ -412,8 +570,18 @@ GRAG_API hipError_t grag_moe_route(const void* h, int ld, const float* wr, int W
   if (E < 1 || R < E || R > RT_MAXR || top < 1 || top > RT_MAXTOP || top > E || ngroups < 1 || E % ngroups ||
       keep < 1 || keep > ngroups)
     return hipErrorInvalidValue;
-  DT_DISPATCH(dt, hipLaunchKernelGGL(moe_route_kernel<T>, dim3((T_ + RT_TOK - 1) / RT_TOK), dim3(256), 0, st,
-                                     (const T*)h, ld, wr, W, E, R, top, ngroups, keep, ids, wts, sgate, T_);)
+  const size_t bytes = ((size_t)(RT_TOK + R) * RT_LD + (size_t)RT_TOK * (R + 1)) * sizeof(float);
+  const int vec = W % 8 == 0 && ld % 8 == 0 && (reinterpret_cast<uintptr_t>(h) & 15) == 0 &&
+                  (reinterpret_cast<uintptr_t>(wr) & 15) == 0;
+  DT_DISPATCH(dt, {
+    if (bytes > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_route_kernel<T>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(moe_route_kernel<T>, dim3((T_ + RT_TOK - 1) / RT_TOK), dim3(256), bytes, st, (const T*)h, ld, wr,
+                       W, E, R, top, ngroups, keep, ids, wts, sgate, T_, vec);
+  })
   return hipGetLastError();
 }
 
@@ -433,6 +601,18 @@ GRAG_API hipError_t grag_moe_gemm(const void* a, int lda, const void* w, const i
   if (tiles > 65535 || E < 1 || top < 1) return hipErrorInvalidValue;
   const dim3 grid((N + MG_N - 1) / MG_N, tiles);
   auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (dt == 0 && K % 8 == 0 && lda % 8 == 0 && al16(a) && al16(w) && rows >= 48 * E) {
+    // prompt-sized row counts (half a large tile per expert on average, or more): the 128 x 128 tiles
+    const int btiles = (rows + 127) / 128 + E;
+    const dim3 bgrid((N + 127) / 128, btiles);
+    if (gated)
+      hipLaunchKernelGGL(moe_gemm_big_kernel<1>, bgrid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,
+                         order, E, top, N, K, (bf16*)out, ldo);
+    else
+      hipLaunchKernelGGL(moe_gemm_big_kernel<0>, bgrid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,
+                         order, E, top, N, K, (bf16*)out, ldo);
+    return hipGetLastError();
+  }
   if (dt == 0 && K % 8 == 0 && lda % 8 == 0 && al16(a) && al16(w)) {
     if (gated)
       hipLaunchKernelGGL(moe_gemm_mfma_kernel<1>, grid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,

@@ -87,7 +87,7 @@ def experts_case(device, dtype, tol):
     from githubrepostorag_amd.ops.moe import moe_experts
 
     g = torch.Generator().manual_seed(3)
-    for T, W, F, E, top in ((9, 48, 20, 6, 2), (70, 64, 40, 5, 3), (3, 40, 24, 4, 4), (1, 33, 7, 3, 1)):
+    for T, W, F, E, top in ((9, 48, 20, 6, 2), (70, 64, 40, 5, 3), (3, 40, 24, 4, 4), (1, 33, 7, 3, 1), (200, 136, 40, 3, 2)):
         h = torch.randn(T, W, generator=g).to(dtype)
         wgu = (torch.randn(E, 2 * F, W, generator=g) / W ** 0.5).to(dtype)
         wd = (torch.randn(E, W, F, generator=g) / F ** 0.5).to(dtype)

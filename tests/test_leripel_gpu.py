@@ -42,7 +42,9 @@ def test_router_alone(dtype):
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 0.02)])
 def test_experts_alone(dtype, tol):
-    T.experts_case("cuda", dtype, tol)  # (fp32: the plain tiles; bf16: the matrix-core tiles, K and F multiples of 8)
+    # fp32: the plain tiles; bf16: the matrix-core tiles where the sizes are multiples of 8, small and (the last case,
+    # 400 rows over 3 experts) large ones
+    T.experts_case("cuda", dtype, tol)
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 0.08)])
