@@ -27,6 +27,66 @@ constexpr int RT_LD = RT_KC + 4;  // LDS row stride (floats): 16-byte rows, bank
 constexpr int RT_MAXR = 256;  // logit rows (experts + the shared gate's row) at most
 constexpr int RT_MAXTOP = 16;
 
+// One token's choice from its logits z [R] (overwritten): scores = softmax of the first E; the `keep` best groups
+// (a group's score is its best expert's) are open; the best `top` experts of the open groups, by falling score, ties
+// to the lower index, weighted by their scores as they are; row E (if any) is the shared expert's gate logit.
+__device__ void route_select(float* z, int E, int R, int top, int ngroups, int keep, int t, int* __restrict__ ids,
+                             float* __restrict__ wts, float* __restrict__ sgate) {
+  if (R > E && sgate != nullptr) sgate[t] = 1.f / (1.f + expf(-z[E]));
+  float mx = -INFINITY;
+  for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
+  float sum = 0.f;
+  for (int e = 0; e < E; ++e) sum += expf(z[e] - mx);
+  const float inv = 1.f / sum;
+  // the open groups: `keep` times, the best group not yet taken (by its best logit: softmax keeps the order)
+  const int per = E / ngroups;
+  unsigned long long open_lo = 0, open_hi = 0, open_2 = 0, open_3 = 0;  // bit g: group g is open (up to 256 groups)
+  auto is_open = [&](int g) {
+    const unsigned long long wbits = g < 64 ? open_lo : g < 128 ? open_hi : g < 192 ? open_2 : open_3;
+    return (wbits >> (g & 63)) & 1ull;
+  };
+  for (int n = 0; n < keep; ++n) {
+    int bg = -1;
+    float bv = -INFINITY;
+    for (int g = 0; g < ngroups; ++g) {
+      if (is_open(g)) continue;
+      float gv = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) gv = fmaxf(gv, z[e]);
+      if (bg < 0 || gv > bv) {
+        bg = g;
+        bv = gv;
+      }
+    }
+    if (bg < 0) break;
+    const unsigned long long bit = 1ull << (bg & 63);
+    if (bg < 64) open_lo |= bit;
+    else if (bg < 128) open_hi |= bit;
+    else if (bg < 192) open_2 |= bit;
+    else open_3 |= bit;
+  }
+  // the best `top` experts of the open groups; a taken expert's logit is overwritten with -inf
+  for (int n = 0; n < top; ++n) {
+    int be = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      if (!is_open(e / per)) continue;
+      const float v = z[e];
+      if (v > bv || (be < 0 && v > -INFINITY)) {
+        be = e;
+        bv = v;
+      }
+    }
+    if (be < 0) {  // fewer open experts than `top`: the rest of the choices carry no weight
+      ids[(size_t)t * top + n] = 0;
+      wts[(size_t)t * top + n] = 0.f;
+      continue;
+    }
+    ids[(size_t)t * top + n] = be;
+    wts[(size_t)t * top + n] = expf(bv - mx) * inv;
+    z[be] = -INFINITY;
+  }
+}
+
 // h [T][ld] (the normed layer input); wr [R][W] fp32, rows 0 .. E-1 the experts, row E (R = E + 1) the shared expert's
 // gate.  ids [T][top] int32, wts [T][top] fp32 (the chosen experts by falling score; ties to the lower index),
 // sgate [T] fp32 = sigmoid(row E's logit).  grid (ceil(T / RT_TOK)), 256 threads: thread (token tid % 16, part
@@ -116,61 +176,48 @@ moe_route_kernel(const T* __restrict__ h, int ld, const float* __restrict__ wr, 
     if (part + 16 * j < R) lgs[tok * (R + 1) + part + 16 * j] = acc[j];
   __syncthreads();
   if (threadIdx.x >= RT_TOK || t0 + threadIdx.x >= T_) return;
-  float* z = lgs + threadIdx.x * (R + 1);
-  const int t = t0 + threadIdx.x;
-  if (R > E && sgate != nullptr) sgate[t] = 1.f / (1.f + expf(-z[E]));
-  float mx = -INFINITY;
-  for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
-  float sum = 0.f;
-  for (int e = 0; e < E; ++e) sum += expf(z[e] - mx);
-  const float inv = 1.f / sum;
-  // the open groups: `keep` times, the best group not yet taken (by its best logit: softmax keeps the order)
-  const int per = E / ngroups;
-  unsigned long long open_lo = 0, open_hi = 0, open_2 = 0, open_3 = 0;  // bit g: group g is open (up to 256 groups)
-  auto is_open = [&](int g) {
-    const unsigned long long wbits = g < 64 ? open_lo : g < 128 ? open_hi : g < 192 ? open_2 : open_3;
-    return (wbits >> (g & 63)) & 1ull;
-  };
-  for (int n = 0; n < keep; ++n) {
-    int bg = -1;
-    float bv = -INFINITY;
-    for (int g = 0; g < ngroups; ++g) {
-      if (is_open(g)) continue;
-      float gv = -INFINITY;
-      for (int e = g * per; e < (g + 1) * per; ++e) gv = fmaxf(gv, z[e]);
-      if (bg < 0 || gv > bv) {
-        bg = g;
-        bv = gv;
+  route_select(lgs + threadIdx.x * (R + 1), E, R, top, ngroups, keep, t0 + threadIdx.x, ids, wts, sgate);
+}
+
+// A few tokens (decode rows): one workgroup per token, one wave per logit row (rows w, w + 4, ...), the lanes split the
+// row's columns (8 consecutive ones per lane and step when `vec`), so the row's loads are all in flight at once and
+// the sum is a wave reduction: the latency of a step no longer scales with the model width.
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_route_rows_kernel(const T* __restrict__ h, int ld, const float* __restrict__ wr, int W, int E, int R, int top,
+                      int ngroups, int keep, int* __restrict__ ids, float* __restrict__ wts,
+                      float* __restrict__ sgate, int vec) {
+  __shared__ float z[RT_MAXR + 1];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const T* hr = h + (size_t)t * ld;
+  for (int r = wid; r < R; r += 4) {
+    const float* w = wr + (size_t)r * W;
+    float a = 0.f;
+    if (vec) {
+      for (int k = lane * 8; k < W; k += 512) {
+        float hv[8];
+        if (sizeof(T) == 2) {
+          const bf16x8_t v = *reinterpret_cast<const bf16x8_t*>(hr + k);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) hv[i] = bits2f(v[i]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) hv[i] = ldm(hr + k + i);
+        }
+        const f32x4_t w0 = *reinterpret_cast<const f32x4_t*>(w + k), w1 = *reinterpret_cast<const f32x4_t*>(w + k + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a = fmaf(hv[i], w0[i], a);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a = fmaf(hv[4 + i], w1[i], a);
       }
+    } else {
+      for (int k = lane; k < W; k += 64) a = fmaf(ldm(hr + k), w[k], a);
     }
-    if (bg < 0) break;
-    const unsigned long long bit = 1ull << (bg & 63);
-    if (bg < 64) open_lo |= bit;
-    else if (bg < 128) open_hi |= bit;
-    else if (bg < 192) open_2 |= bit;
-    else open_3 |= bit;
+    a = wave_sum(a);
+    if (lane == 0) z[r] = a;
   }
-  // the best `top` experts of the open groups; a taken expert's logit is overwritten with -inf
-  for (int n = 0; n < top; ++n) {
-    int be = -1;
-    float bv = -INFINITY;
-    for (int e = 0; e < E; ++e) {
-      if (!is_open(e / per)) continue;
-      const float v = z[e];
-      if (v > bv || (be < 0 && v > -INFINITY)) {
-        be = e;
-        bv = v;
-      }
-    }
-    if (be < 0) {  // fewer open experts than `top`: the rest of the choices carry no weight
-      ids[(size_t)t * top + n] = 0;
-      wts[(size_t)t * top + n] = 0.f;
-      continue;
-    }
-    ids[(size_t)t * top + n] = be;
-    wts[(size_t)t * top + n] = expf(bv - mx) * inv;
-    z[be] = -INFINITY;
-  }
+  __syncthreads();
+  if (threadIdx.x == 0) route_select(z, E, R, top, ngroups, keep, t, ids, wts, sgate);
 }
 
 // ------------------------------------------------------------------------------------------------ alignment
@@ -573,6 +620,11 @@ GRAG_API hipError_t grag_moe_route(const void* h, int ld, const float* wr, int W
   const size_t bytes = ((size_t)(RT_TOK + R) * RT_LD + (size_t)RT_TOK * (R + 1)) * sizeof(float);
   const int vec = W % 8 == 0 && ld % 8 == 0 && (reinterpret_cast<uintptr_t>(h) & 15) == 0 &&
                   (reinterpret_cast<uintptr_t>(wr) & 15) == 0;
+  if (T_ <= 128) {  // decode rows, short portions
+    DT_DISPATCH(dt, hipLaunchKernelGGL(moe_route_rows_kernel<T>, dim3(T_), dim3(256), 0, st, (const T*)h, ld, wr, W, E, R,
+                                       top, ngroups, keep, ids, wts, sgate, vec);)
+    return hipGetLastError();
+  }
   DT_DISPATCH(dt, {
     if (bytes > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_route_kernel<T>),
