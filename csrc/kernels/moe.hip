@@ -595,6 +595,72 @@ residual_rmsnorm_kernel(float* __restrict__ x, float keep, const T* __restrict__
   }
 }
 
+// the same with 16-byte accesses of x (8-byte ones of bf16 rows): H a multiple of 4, H <= 4 * 256 * RBV_PER, every
+// pointer 16-byte aligned (raw_ld a multiple of 4 too).  A thread keeps its RBV_PER groups of four in registers.
+constexpr int RBV_PER = 4;
+template <typename T> __device__ __forceinline__ f32x4_t ld4(const T* p);
+template <> __device__ __forceinline__ f32x4_t ld4<float>(const float* p) { return *reinterpret_cast<const f32x4_t*>(p); }
+template <> __device__ __forceinline__ f32x4_t ld4<bf16>(const bf16* p) {
+  const bf16x4_t v = *reinterpret_cast<const bf16x4_t*>(p);
+  return f32x4_t{bits2f(v[0]), bits2f(v[1]), bits2f(v[2]), bits2f(v[3])};
+}
+template <typename T> __device__ __forceinline__ void st4(T* p, f32x4_t v);
+template <> __device__ __forceinline__ void st4<float>(float* p, f32x4_t v) { *reinterpret_cast<f32x4_t*>(p) = v; }
+template <> __device__ __forceinline__ void st4<bf16>(bf16* p, f32x4_t v) {
+  *reinterpret_cast<bf16x4_t*>(p) = bf16x4_t{f2bits(v[0]), f2bits(v[1]), f2bits(v[2]), f2bits(v[3])};
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+residual_rmsnorm_vec_kernel(float* __restrict__ x, float keep, const T* __restrict__ a, const T* __restrict__ b,
+                            const float* __restrict__ bcoef, const T* __restrict__ e, const float* __restrict__ ecoef,
+                            int K, const float* __restrict__ w, float eps, T* __restrict__ out, T* __restrict__ raw,
+                            int raw_ld, int H) {
+  __shared__ float red[16];
+  const size_t t = blockIdx.x, row = t * H;
+  const float bc = b ? (bcoef ? bcoef[t] : 1.f) : 0.f;
+  f32x4_t v[RBV_PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < RBV_PER; ++u) {
+    const int i = (threadIdx.x + 256 * u) * 4;
+    v[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (i < H) {
+      f32x4_t y = a ? ld4(a + row + i) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+      f32x4_t f = b ? bc * ld4(b + row + i) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int k = 0; k < K; ++k) {
+        const float c = ecoef[t * K + k];
+        const f32x4_t ev = ld4(e + (t * K + k) * H + i);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) f[r] = fmaf(c, ev[r], f[r]);
+      }
+      y += f;
+      f32x4_t nx = y;
+      if (keep != 0.f) {
+        const f32x4_t xv = *reinterpret_cast<const f32x4_t*>(x + row + i);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) nx[r] = keep * xv[r] + y[r];
+      }
+      *reinterpret_cast<f32x4_t*>(x + row + i) = nx;
+      v[u] = nx;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ss = fmaf(nx[r], nx[r], ss);
+      if (raw) st4(raw + t * raw_ld + i, nx);
+    }
+  }
+  if (out == nullptr) return;
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+  for (int u = 0; u < RBV_PER; ++u) {
+    const int i = (threadIdx.x + 256 * u) * 4;
+    if (i < H) {
+      const f32x4_t wv = *reinterpret_cast<const f32x4_t*>(w + i);
+      st4(out + row + i, f32x4_t{v[u][0] * r * wv[0], v[u][1] * r * wv[1], v[u][2] * r * wv[2], v[u][3] * r * wv[3]});
+    }
+  }
+}
+
 }  // namespace grag
 
 using namespace grag;
@@ -691,6 +757,14 @@ GRAG_API hipError_t grag_residual_rmsnorm(float* x, float keep, const void* a, c
   if (T_ <= 0) return hipSuccess;
   if (K < 0 || (K > 0 && (e == nullptr || ecoef == nullptr)) || (out != nullptr && w == nullptr))
     return hipErrorInvalidValue;
+  auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (H % 4 == 0 && H <= 4 * 256 * RBV_PER && al16(x) && al16(a) && al16(b) && al16(e) && al16(w) && al16(out) &&
+      al16(raw) && raw_ld % 8 == 0) {
+    DT_DISPATCH(dt, hipLaunchKernelGGL(residual_rmsnorm_vec_kernel<T>, dim3(T_), dim3(256), 0, st, x, keep,
+                                       (const T*)a, (const T*)b, bcoef, (const T*)e, ecoef, e ? K : 0, w, eps, (T*)out,
+                                       (T*)raw, raw_ld, H);)
+    return hipGetLastError();
+  }
   DT_DISPATCH(dt, hipLaunchKernelGGL(residual_rmsnorm_kernel<T>, dim3(T_), dim3(256), 0, st, x, keep, (const T*)a,
                                      (const T*)b, bcoef, (const T*)e, ecoef, e ? K : 0, w, eps, (T*)out, (T*)raw,
                                      raw_ld, H);)
