@@ -61,8 +61,8 @@ def router_case(device, dtype):
 
     g = torch.Generator().manual_seed(2)
     # (37 tokens: the kernel of decode rows and short portions; 150: the tiled kernel of prompts)
-    for E, top, groups, keep, W, T in ((6, 2, 3, 2, 40, 37), (16, 4, 4, 3, 64, 150), (8, 8, 1, 1, 24, 37), (9, 1, 9, 1, 16, 37),
-                                       (12, 3, 4, 4, 33, 37), (12, 3, 4, 4, 33, 131), (16, 4, 4, 3, 264, 9)):
+    for E, top, groups, keep, W, T in ((6, 2, 3, 2, 40, 37), (20, 4, 5, 3, 64, 150), (8, 8, 1, 1, 24, 37), (9, 1, 9, 1, 16, 37),
+                                       (12, 3, 4, 4, 33, 37), (12, 3, 4, 4, 33, 131), (24, 5, 6, 2, 264, 9)):
         h = torch.randn(T, W, generator=g).to(dtype)
         wr = (torch.randn(E + 1, W, generator=g) * 0.7).to(torch.bfloat16).float()
         ids, wts, gate = moe_route(h.to(device), wr.to(device), E, top, groups, keep)
