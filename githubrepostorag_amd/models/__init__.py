@@ -22,6 +22,10 @@ def build_decoder(cfg, **kw):
         from .leripel import LeripelModel
 
         return LeripelModel(cfg, **kw)
+    if cfg.arch == "pubulix":
+        from .pubulix import PubulixModel
+
+        return PubulixModel(cfg, **kw)
     from .qwen2 import Qwen2Model
 
     return Qwen2Model(cfg, **kw)

@@ -135,6 +135,27 @@ class LatentAttnSpec:
     q_rank: int
     scale: float
     rot_base: float
+    window: int = 0  # > 0: a query sees itself and the window - 1 positions before it
+    kv_from: int | None = None  # the layer whose cached latent and rotated key part this layer attends to
+    q_latent: bool = True  # False: queries straight from the layer input (no query latent)
+    sink: bool = False  # one learned key-less logit per head in the softmax's denominator
+    gate: bool = False  # the concatenated heads are multiplied by the sigmoid of a projection of the input
+    interleaved: bool = False  # rotary pairs (2i, 2i + 1) instead of (i, i + rot_dim / 2)
+
+
+@dataclass(frozen=True)
+class CappedAttnSpec:
+    """Sliding-window softmax attention, GQA, partial rotary on halves, scores capped by softcap * tanh(s / softcap)
+    (softcap 0: no cap; window 0: plain causal)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int
+    softcap: float
+    rot_dims: int
+    rot_base: float
 
 
 @dataclass(frozen=True)
@@ -184,6 +205,8 @@ class MoESpec:
     groups: int
     keep: int
     shared_ff: int
+    limit: float | None = None  # clamped units g sigmoid(1.702 g) (u + 1), g = min(gate, limit), u = clamp(up, +-limit)
+    table: bool = False  # no router: a [vocab, top] table names every token id's experts, each weighs 1 / top
 
 
 @dataclass(frozen=True)
@@ -194,7 +217,7 @@ class MixerSpec:
     left_scale: float = 1.0
     right_scale: float = 1.0
     width: int = 0  # mingru state width
-    spec: RetentionSpec | WindowAttnSpec | LatentAttnSpec | ChunkAttnSpec | SSMSpec | None = None  # single-mixer kinds
+    spec: RetentionSpec | WindowAttnSpec | LatentAttnSpec | ChunkAttnSpec | CappedAttnSpec | SSMSpec | None = None  # single-mixer kinds
 
 
 @dataclass(frozen=True)
@@ -224,6 +247,10 @@ class HybridConfig:
     max_position: int = 1 << 20  # the design has no position limit of its own: the engine's max_model_len bounds it
     tie_word_embeddings: bool = False
     streams: int = 1  # residual streams (hyper-connections); 1 = the plain residual sum
+    embed_scale: float = 1.0  # the embedding rows are multiplied by this
+    residual_mult: float = 1.0  # every sublayer's output is multiplied by this before it joins the residual
+    logit_softcap: float = 0.0  # > 0: logits <- cap * tanh(logits / cap)
+    conv_taps: int = 0  # > 0: every mixer reads h + conv(h), a causal per-channel convolution of this many taps
 
     @property
     def num_layers(self) -> int:
@@ -246,6 +273,21 @@ class HybridConfig:
 
     def param_count(self) -> int:
         H = self.hidden_size
+        if self.arch == "pubulix":
+            n = 2 * self.vocab_size * H + 1
+            for L in self.layers:
+                m, a = L.mixer.kind, L.mixer.spec
+                n += 1 + H * self.conv_taps + H * H + H
+                if m == "attention":
+                    n += H * (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim)) + a.heads * a.vdim * H
+                else:
+                    n += H * a.heads * (a.dim + a.rot_dim) + a.kv_rank * a.heads * (a.dim + a.vdim) + a.heads
+                    n += 2 * H * a.heads * a.vdim
+                    if a.kv_from is None:
+                        n += H * (a.kv_rank + a.rot_dim) + a.kv_rank
+                if L.mlp is not None:
+                    n += 1 + H * H + H + L.mlp.experts * 3 * H * L.mlp.ff
+            return n
         if self.arch == "leripel":
             n = 2 * self.vocab_size * H + H + (2 * H * H if self.loop_stop > self.loop_start else 0)
             for L in self.layers:
@@ -522,6 +564,112 @@ def leripel_config(name: str, vocab: int, width: int, pattern: str, *, heads: in
                         arch="leripel")
 
 
+def pubulix_config_from_dict(d: dict, name: str = "pubulix") -> HybridConfig:
+    """The Pubulix design's config.json: a layer list of "attention" (capped sliding-window GQA) and
+    "latent_attention" (sliding-window attention over a cached latent, with a sink and an output gate; a layer may
+    attend to an earlier layer's cache) mixers, each with an optional table-routed mixture of clamped experts; a
+    scalar-weight RMS norm, an input convolution in front of every mixer, sigmoid-gated residual branches.  Every
+    size and constant is read from it."""
+    layers = []
+    for i, e in enumerate(d["layers"]):
+        kind, m = e["type"], e["mixer"]
+        rot = m.get("rot") or {"dims": 0, "base": 1.0}
+        mask = m.get("mask") or {"size": 0}
+        if kind == "attention":
+            a = CappedAttnSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]),
+                               int(m.get("vdim", m["dim"])), float(m["scale"]), int(mask.get("size", 0)),
+                               float(m.get("softcap") or 0.0), int(rot["dims"]), float(rot.get("base", 1.0)))
+            if a.heads % a.kv_heads or a.rot_dims % 2 or a.rot_dims > a.dim or a.window < 0 or a.softcap < 0:
+                raise ValueError(f"bad attention sizes {m}")
+        elif kind == "latent_attention":
+            src = m.get("kv_from")
+            a = LatentAttnSpec(int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"]), 0,
+                               float(m["scale"]), float(rot.get("base", 10000.0)), int(mask.get("size", 0)),
+                               None if src is None else int(src), q_latent=False, sink=True, gate=True,
+                               interleaved=True)
+            if a.rot_dim % 2 or int(rot.get("dims", a.rot_dim)) != a.rot_dim or a.window < 0:
+                raise ValueError(f"bad latent attention sizes {m} (the rotated part is rotated whole)")
+            if a.kv_from is not None:
+                o = layers[a.kv_from].mixer if 0 <= a.kv_from < i else None
+                if (o is None or o.kind != "latent_attention" or o.spec.kv_from is not None
+                        or (o.spec.kv_rank, o.spec.rot_dim, o.spec.rot_base) != (a.kv_rank, a.rot_dim, a.rot_base)):
+                    raise ValueError(f"layer {i}: kv_from {a.kv_from} names no earlier latent layer with a cache of "
+                                     "its own and the same latent size and rotation")
+        else:
+            raise ValueError(f"unknown mixer type {kind!r}")
+        f = e.get("mlp")
+        if f is None:
+            mlp = None
+        elif f.get("kind", "moe") == "moe":
+            r = f["router"]
+            lim = f["expert"].get("limit")
+            mlp = MoESpec("moe", int(f["expert"]["ff"]), int(r["experts"]), int(r["top"]), 1, 1, 0,
+                          None if lim is None else float(lim), table=True)
+            if not 1 <= mlp.top <= mlp.experts:
+                raise ValueError(f"bad expert table sizes {r}")
+        else:
+            raise ValueError(f"unknown feed-forward kind {f.get('kind')!r}")
+        layers.append(HybridLayerSpec(MixerSpec(kind, spec=a), mlp))
+    taps = int((d.get("canon") or {}).get("taps", 0))
+    if taps < 0:
+        raise ValueError("canon.taps < 0")
+    return HybridConfig(name, int(d["vocab"]), int(d["width"]), float(d["norm"]["eps"]), tuple(layers), arch="pubulix",
+                        embed_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
+                        residual_mult=float(d.get("residual_mult", 1.0)),
+                        logit_softcap=float(d.get("logit_softcap") or 0.0), conv_taps=taps)
+
+
+def pubulix_config_to_dict(cfg: HybridConfig) -> dict:
+    """Back to the config.json form (checkpoint export, tests)."""
+    layers = []
+    for L in cfg.layers:
+        a, kind = L.mixer.spec, L.mixer.kind
+        if kind == "attention":
+            m = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale,
+                 "softcap": a.softcap, "mask": {"size": a.window}, "rot": {"dims": a.rot_dims, "base": a.rot_base}}
+        else:
+            m = {"heads": a.heads, "dim": a.dim, "rot_dim": a.rot_dim, "vdim": a.vdim, "kv_rank": a.kv_rank,
+                 "scale": a.scale, "mask": {"size": a.window}, "rot": {"dims": a.rot_dim, "base": a.rot_base}}
+            if a.kv_from is not None:
+                m["kv_from"] = a.kv_from
+        f = L.mlp
+        mlp = None if f is None else {"kind": "moe", "expert": {"ff": f.ff, "limit": f.limit},
+                                      "router": {"experts": f.experts, "top": f.top}}
+        layers.append({"type": kind, "mixer": m, "mlp": mlp})
+    return {"architecture": "Pubulix", "vocab": cfg.vocab_size, "width": cfg.hidden_size,
+            "norm": {"eps": cfg.norm_eps}, "canon": {"taps": cfg.conv_taps}, "embedding": {"scale": cfg.embed_scale},
+            "residual_mult": cfg.residual_mult, "logit_softcap": cfg.logit_softcap, "layers": layers}
+
+
+def pubulix_config(name: str, vocab: int, width: int, pattern: str, *, heads: int, kv_heads: int, dim: int,
+                   window: int = 1024, softcap: float = 50.0, rot_dims: int | None = None, lat_heads: int | None = None,
+                   lat_dim: int | None = None, lat_vdim: int | None = None, kv_rank: int = 256, rot_dim: int = 32,
+                   lat_window: int = 2048, experts: int = 16, top: int = 2, ff: int = 1024, limit: float = 7.0,
+                   taps: int = 4, eps: float = 1e-5, embed_scale: float = 1.0, residual_mult: float = 1.0,
+                   logit_softcap: float = 30.0, moe: bool = True) -> HybridConfig:
+    """A regular Pubulix stack for benches and plumbing tests.  ``pattern``: one letter per layer, a = capped
+    sliding-window attention, l = latent attention with a cache of its own, s = latent attention over the cache of
+    the nearest "l" before it; every layer carries the same table-routed experts."""
+    lh, ld, lv = lat_heads or heads, lat_dim or dim, lat_vdim or dim
+    mlp = MoESpec("moe", ff, experts, top, 1, 1, 0, limit, table=True) if moe else None
+    layers, last = [], None
+    for i, c in enumerate(pattern):
+        if c == "a":
+            spec = CappedAttnSpec(heads, kv_heads, dim, dim, dim ** -0.5, window, softcap,
+                                  dim if rot_dims is None else rot_dims, 1e4)
+            layers.append(HybridLayerSpec(MixerSpec("attention", spec=spec), mlp))
+            continue
+        if c == "l":
+            last = i
+        elif last is None:
+            raise ValueError("an 's' layer needs an 'l' layer before it")
+        spec = LatentAttnSpec(lh, ld, rot_dim, lv, kv_rank, 0, (ld + rot_dim) ** -0.5, 1e4, lat_window,
+                              last if c == "s" else None, q_latent=False, sink=True, gate=True, interleaved=True)
+        layers.append(HybridLayerSpec(MixerSpec("latent_attention", spec=spec), mlp))
+    return HybridConfig(name, vocab, width, eps, tuple(layers), arch="pubulix", embed_scale=embed_scale,
+                        residual_mult=residual_mult, logit_softcap=logit_softcap, conv_taps=taps)
+
+
 def zofesun_config(name: str, vocab: int, width: int, n_layers: int, *, heads: int, kv_heads: int, dim: int,
                    vdim: int, lin_heads: int, lin_dim: int, lin_vdim: int, ff: int, mingru_every: int = 0,
                    rot_dims: int | None = None, rot_base: float = 10000.0, loop=(0, 0, 1), limit: float = 7.0,
@@ -565,6 +713,16 @@ HYBRIDS = {
     "leripel-7b": leripel_config("leripel-7b", 32768, 3584, "rama", heads=28, kv_heads=4, dim=128, chunk=1024,
                                  ssm_vdim=64, ssm_state=128, experts=16, top=4, groups=(4, 2), ff=3840,
                                  shared_ff=3584),
+    # Pubulix: a plumbing-test size and two bench sizes with the layer shapes of a 1.5B / 7B decoder (the experts'
+    # active width top * ff equals the dense decoders' feed-forward width)
+    "pubulix-tiny": pubulix_config("pubulix-tiny", 320, 96, "alas", heads=4, kv_heads=2, dim=16, window=9, softcap=8.0,
+                                   rot_dims=8, lat_heads=3, lat_dim=8, lat_vdim=12, kv_rank=24, rot_dim=8,
+                                   lat_window=13, experts=6, top=2, ff=40, limit=1.5, taps=3, embed_scale=2.0,
+                                   residual_mult=0.5),
+    "pubulix-1b": pubulix_config("pubulix-1b", 32768, 1536, "alasalas", heads=12, kv_heads=2, dim=128, window=1024,
+                                 lat_heads=12, kv_rank=192, rot_dim=64, lat_window=2048, experts=16, top=4, ff=2240),
+    "pubulix-7b": pubulix_config("pubulix-7b", 32768, 3584, "alas", heads=28, kv_heads=4, dim=128, window=1024,
+                                 lat_heads=28, kv_rank=192, rot_dim=64, lat_window=2048, experts=16, top=4, ff=4736),
 }
 
 
@@ -579,6 +737,8 @@ def config_from_dir(path) -> DecoderConfig | HybridConfig:
         return namudra_config_from_dict(d, Path(path).name or "namudra")
     if arch == "leripel":
         return leripel_config_from_dict(d, Path(path).name or "leripel")
+    if arch == "pubulix":
+        return pubulix_config_from_dict(d, Path(path).name or "pubulix")
     mt = str(d.get("model_type", "")).lower()
     if mt == "gpt2":
         return DecoderConfig(Path(path).name, d["vocab_size"], d["n_embd"], d.get("n_inner") or 4 * d["n_embd"],

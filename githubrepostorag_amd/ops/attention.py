@@ -414,11 +414,12 @@ def varlen_attention(qkv: torch.Tensor, seq_start: torch.Tensor, seq_len: torch.
 
 # ---------------------------------------------------------------------------------------------- sink attention
 def sink_attention_ref(q, k_cache, v_cache, meta: AttnMetadata, scale: float, sinks: torch.Tensor,
-                       head_scale: torch.Tensor | None = None, chunk: int = 0):
+                       head_scale: torch.Tensor | None = None, chunk: int = 0, window: int = 0, softcap: float = 0.0):
     """fp32: q [T, H, d], k_cache [blocks, G, BS, d], v_cache [blocks, G, BS, vd] -> [T, H, vd].  Causal softmax
     whose denominator also holds exp(sinks[h]): one more logit with no key and no value.  ``head_scale`` [H]
     multiplies the scores of head h; ``chunk`` > 0: a query sees only the keys of its own aligned block of that
-    many positions."""
+    many positions; ``window`` > 0: only the keys at most window - 1 positions back; ``softcap`` > 0: the scaled
+    scores go through softcap * tanh(score / softcap)."""
     T, H, d = q.shape
     G, BS, vd = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
     R = H // G
@@ -435,11 +436,15 @@ def sink_attention_ref(q, k_cache, v_cache, meta: AttnMetadata, scale: float, si
         sc = torch.einsum("phd,khd->hpk", q[a:b].float(), K) * scale
         if head_scale is not None:
             sc = sc * head_scale.float().view(H, 1, 1)
+        if softcap > 0:
+            sc = softcap * torch.tanh(sc / softcap)
         pos = torch.arange(ctx - ql, ctx, device=q.device)[:, None]
         keys = torch.arange(ctx, device=q.device)[None, :]
         hidden = keys > pos
         if chunk > 0:
             hidden = hidden | (keys < pos - pos % chunk)
+        if window > 0:
+            hidden = hidden | (keys < pos - (window - 1))
         sc = sc.masked_fill(hidden[None], float("-inf"))
         sk = sinks.float().view(H, 1, 1).expand(H, ql, 1)
         p = torch.softmax(torch.cat([sc, sk], dim=-1), dim=-1)[..., :ctx]
@@ -463,7 +468,7 @@ def no_sinks(H: int, device) -> torch.Tensor:
 def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, meta: AttnMetadata, scale: float,
                    sinks: torch.Tensor | None, out: torch.Tensor | None = None, out_scale: float = 1.0,
                    head_scale: torch.Tensor | None = None, head_gate: torch.Tensor | None = None,
-                   chunk: int = 0) -> torch.Tensor:
+                   chunk: int = 0, window: int = 0, softcap: float = 0.0) -> torch.Tensor:
     """Paged causal attention with a sink term, key size != value size allowed: q [T, H, d] -> out [T, H*vd]
     (``out`` may be a column slice of a wider buffer), multiplied by ``out_scale``.  Prefill chunks run the
     tiled kernel, decode rows (one query per sequence) the decode kernel; a mixed step runs both.  ``sinks``
@@ -471,7 +476,9 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     ``head_scale`` [H] fp32: a temperature per head (multiplies ``scale``).  ``chunk`` > 0: block-local attention,
     a query at position i sees key j <= i only when floor(j / chunk) == floor(i / chunk); positions count from the
     start of the sequence, however the prompt was cut.  ``head_gate`` [T, H] (a column slice of a fused
-    projection is fine): head h's output is multiplied by sigmoid(head_gate[t, h]) as it is stored."""
+    projection is fine): head h's output is multiplied by sigmoid(head_gate[t, h]) as it is stored.
+    ``window`` > 0: sliding-window attention, a query at position i sees key j only when 0 <= i - j < window.
+    ``softcap`` > 0: score <- softcap * tanh(score / softcap) after the scaling, before the softmax."""
     if sinks is None:
         sinks = no_sinks(q.shape[1], q.device)
     T, H, d = q.shape
@@ -485,14 +492,14 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                              slot_mapping=meta.slot_mapping, max_q_len=meta.max_q_len, num_seqs=meta.num_seqs,
                              num_tokens=Tp)
         sink_attention(q[:Tp], k_cache, v_cache, pmeta, scale, sinks, out[:Tp], out_scale, head_scale,
-                       None if head_gate is None else head_gate[:Tp], chunk)
+                       None if head_gate is None else head_gate[:Tp], chunk, window, softcap)
         sink_attention(q[Tp:], k_cache, v_cache, dmeta, scale, sinks, out[Tp:], out_scale, head_scale,
-                       None if head_gate is None else head_gate[Tp:], chunk)
+                       None if head_gate is None else head_gate[Tp:], chunk, window, softcap)
         return out
     if T == 0:
         return out
     if not q.is_cuda:
-        o = sink_attention_ref(q, k_cache, v_cache, meta, scale, sinks, head_scale, chunk) * out_scale
+        o = sink_attention_ref(q, k_cache, v_cache, meta, scale, sinks, head_scale, chunk, window, softcap) * out_scale
         if head_gate is not None:
             o = o * torch.sigmoid(head_gate.float())[:, :, None]
         out.copy_(o.reshape(T, H * vd))
@@ -500,7 +507,8 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     assert q.is_contiguous() and out.stride(1) == 1 and sinks.dtype == torch.float32 and k_cache.is_contiguous()
     assert head_scale is None or (head_scale.dtype == torch.float32 and head_scale.numel() == H)
     assert head_gate is None or (head_gate.dtype == q.dtype and head_gate.stride(1) == 1 and head_gate.shape == (T, H))
-    extra = (ptr(head_scale), ptr(head_gate), 0 if head_gate is None else head_gate.stride(0), int(chunk))
+    extra = (ptr(head_scale), ptr(head_gate), 0 if head_gate is None else head_gate.stride(0), int(chunk),
+             int(window), float(softcap))
     # value rows may be the head of wider rows (a view [..., :vd] of a cache whose rows hold more: latent attention
     # reads its values out of its key rows): v_ld is the row stride, the block / head strides must follow from it
     v_ld = v_cache.stride(2)
@@ -509,7 +517,7 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     if meta.is_decode and meta.max_q_len == 1:
         # key splits (flash-decoding) when the step brings a plan and scratch that holds it
         nsplit = meta.num_splits
-        if 0 < chunk <= 1024:  # a block's keys are few: one workgroup per (sequence, kv head) walks them
+        if 0 < chunk <= 1024 or 0 < window <= 1024:  # the visible keys are few: one workgroup per (sequence, kv head)
             nsplit = 1
         if (nsplit > 1 and (meta.part_o is None or meta.part_ml is None
                             or meta.part_o.numel() < nsplit * meta.num_seqs * H * vd

@@ -282,3 +282,64 @@ def latent_store(ckv: torch.Tensor, cw: torch.Tensor, positions: torch.Tensor, t
          ptr(slot_mapping), ptr(q), ptr(k_cache), T, H, R, r, BS, k_cache.shape[0] * BS, float(eps),
          0 if ckv.dtype == torch.bfloat16 else 1)
     return q
+
+
+def latent_rope_store(proj: torch.Tensor, qoff: int, coff: int | None, cw: torch.Tensor | None,
+                      positions: torch.Tensor, table: torch.Tensor, slot_mapping: torch.Tensor,
+                      k_cache: torch.Tensor, H: int, eps: float, interleaved: bool = False) -> torch.Tensor:
+    """Latent attention's cache row and queries out of one fused projection ``proj`` [T, ld].  Columns qoff ..: H
+    query heads of R + r columns each (R against the latent, r = the width of ``table``, a rope_table, to rotate);
+    returned as q [T, H, R + r] with the last r columns of every head rotated by ``positions``.  Columns coff ..
+    (``coff`` None: this layer reads another layer's cache and stores nothing): a latent of R columns and the r
+    columns of the key part all heads share; k_cache [blocks, 1, BS, R + r] <- latent / rms(latent) * cw | rotated
+    part at ``slot_mapping`` (-1: not stored).  Rotation pairs dim i with i + r/2, or 2i with 2i + 1 when
+    ``interleaved`` (pair i turned by the table's angle i); the statistics and the rotation are fp32."""
+    T = proj.shape[0]
+    BS, r = k_cache.shape[2], table.shape[1]
+    R = k_cache.shape[3] - r
+    h2 = r // 2
+
+    if not proj.is_cuda:
+        x = proj.float()
+        cs = table[positions.long()]
+        co, sn = cs[:, :h2], cs[:, h2:]
+
+        def rot(t, co, sn):
+            if interleaved:
+                a, b = t[..., 0::2], t[..., 1::2]
+                return torch.stack([a * co - b * sn, b * co + a * sn], dim=-1).flatten(-2)
+            a, b = t[..., :h2], t[..., h2:]
+            return torch.cat([a * co - b * sn, b * co + a * sn], dim=-1)
+
+        q = x[:, qoff:qoff + H * (R + r)].reshape(T, H, R + r).clone()
+        q[:, :, R:] = rot(q[:, :, R:], co[:, None], sn[:, None])
+        if coff is not None:
+            c = x[:, coff:coff + R]
+            c = c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps) * cw.float()
+            kr = rot(x[:, coff + R:coff + R + r], co, sn)
+            ok = slot_mapping >= 0
+            sl = slot_mapping[ok].long()
+            k_cache[sl // BS, 0, sl % BS] = torch.cat([c, kr], -1)[ok].to(k_cache.dtype)
+        return q.to(proj.dtype)
+    assert proj.stride(1) == 1 and k_cache.dtype == proj.dtype and k_cache.is_contiguous() and k_cache.shape[1] == 1
+    assert R > 0 and r % 2 == 0 and table.dtype == torch.float32
+    assert coff is None or (cw is not None and cw.dtype == torch.float32 and cw.numel() == R)
+    assert qoff + H * (R + r) <= proj.shape[1] and (coff is None or coff + R + r <= proj.shape[1])
+    q = torch.empty(T, H, R + r, dtype=proj.dtype, device=proj.device)
+    call("grag_latent_rope_store", ptr(proj), proj.stride(0), qoff, -1 if coff is None else coff, ptr(cw),
+         ptr(positions), ptr(table), table.shape[0], ptr(slot_mapping), ptr(q), ptr(k_cache), T, H, R, r, BS,
+         k_cache.shape[0] * BS, float(eps), 0 if proj.dtype == torch.bfloat16 else 1, 1 if interleaved else 0)
+    return q
+
+
+def tanh_cap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """In place: x <- cap * tanh(x / cap), evaluated in fp32 (``cap`` <= 0: x as it is).  x [rows, N], rows may be
+    a column slice of a wider tensor."""
+    if cap <= 0 or x.numel() == 0:
+        return x
+    if not x.is_cuda:
+        x.copy_((cap * torch.tanh(x.float() / cap)).to(x.dtype))
+        return x
+    assert x.dim() == 2 and x.stride(1) == 1
+    call("grag_tanh_cap", ptr(x), x.stride(0), x.shape[0], x.shape[1], float(cap), 0 if x.dtype == torch.bfloat16 else 1)
+    return x

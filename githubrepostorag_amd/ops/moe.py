@@ -1,5 +1,6 @@
 """Mixture-of-experts feed-forward ops (HIP on device tensors, plain fp32 on CPU): the router with group-limited
-top-k choice, and the experts' SiLU-gated units over the chosen (token, expert) pairs.
+top-k choice (or a table that names every token id's experts), and the experts' gated units over the chosen
+(token, expert) pairs; the same grouped GEMM also runs one small matrix per attention head.
 
 The router's logits, scores and weights are fp32.  The experts run as two grouped GEMMs over the pairs sorted by
 expert; their outputs come back in (token, choice) order and are summed, with the router's weights, in fp32 by the
@@ -46,10 +47,26 @@ def moe_route(h: torch.Tensor, wr: torch.Tensor, E: int, top: int, groups: int =
     return ids, wts, gate
 
 
-def moe_experts(h: torch.Tensor, ids: torch.Tensor, wgu: torch.Tensor, wd: torch.Tensor) -> torch.Tensor:
+def moe_table_route(token_ids: torch.Tensor, table: torch.Tensor):
+    """Routing without a router: ``table`` [vocab, top] int32 names the experts of every token id.  Returns
+    (ids [T, top] int32 = the rows of the step's token ids, wts [T, top] fp32 = 1 / top each)."""
+    T, top = token_ids.numel(), table.shape[1]
+    if not table.is_cuda:
+        ids = table[token_ids.long()].to(torch.int32).contiguous()
+        return ids, torch.full((T, top), 1.0 / top, dtype=torch.float32)
+    assert table.dtype == torch.int32 and table.is_contiguous() and token_ids.dtype == torch.int32
+    ids = torch.empty(T, top, dtype=torch.int32, device=table.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=table.device)
+    call("grag_moe_table_route", ptr(token_ids), ptr(table), table.shape[0], top, ptr(ids), ptr(wts), T)
+    return ids, wts
+
+
+def moe_experts(h: torch.Tensor, ids: torch.Tensor, wgu: torch.Tensor, wd: torch.Tensor,
+                limit: float | None = None, alpha: float = 1.0, shift: float = 0.0) -> torch.Tensor:
     """The chosen experts' outputs, unweighted: h [T, W], ids [T, top] int32, ``wgu`` [E, 2F, W] (every expert's gate
     rows, then its up rows), ``wd`` [E, W, F] -> [T, top, W] with out[t, k] = wd[e] (silu(gate_e h_t) * (up_e h_t)),
-    e = ids[t, k]."""
+    e = ids[t, k].  With ``limit`` / ``alpha`` / ``shift`` the unit is g sigmoid(alpha g) (u + shift) with
+    g = min(gate, limit), u = clamp(up, -limit, limit) (``limit`` None: no clamp)."""
     T, W = h.shape
     top = ids.shape[1]
     E, F2, _ = wgu.shape
@@ -61,7 +78,10 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wgu: torch.Tensor, wd: torch
             for k in range(top):
                 e = int(ids[t, k])
                 gu = wgu[e].float() @ x[t]
-                act = (torch.nn.functional.silu(gu[:F]) * gu[F:]).to(h.dtype)  # (the kernels store it in h's type)
+                g, u = gu[:F], gu[F:]
+                if limit is not None:
+                    g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+                act = (g * torch.sigmoid(alpha * g) * (u + shift)).to(h.dtype)  # (the kernels store it in h's type)
                 out[t, k] = wd[e].float() @ act.float()
         return out.to(h.dtype)
     assert h.stride(1) == 1 and wgu.is_contiguous() and wd.is_contiguous() and ids.is_contiguous()
@@ -71,7 +91,44 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wgu: torch.Tensor, wd: torch
     order = torch.empty(n, dtype=torch.int32, device=h.device)
     call("grag_moe_align", ptr(ids), n, E, ptr(offs), ptr(order))
     act = torch.empty(n, F, dtype=h.dtype, device=h.device)
-    call("grag_moe_gemm", ptr(h), h.stride(0), ptr(wgu), ptr(offs), ptr(order), n, E, top, F, W, ptr(act), F, 1, _dt(h))
+    lim = float("inf") if limit is None else float(limit)
+    call("grag_moe_gemm", ptr(h), h.stride(0), ptr(wgu), ptr(offs), ptr(order), n, E, top, F, W, ptr(act), F, 1, _dt(h),
+         lim, float(alpha), float(shift), None, 0)
     out = torch.empty(T, top, W, dtype=h.dtype, device=h.device)
-    call("grag_moe_gemm", ptr(act), F, ptr(wd), ptr(offs), ptr(order), n, E, top, W, F, ptr(out), W, 0, _dt(h))
+    call("grag_moe_gemm", ptr(act), F, ptr(wd), ptr(offs), ptr(order), n, E, top, W, F, ptr(out), W, 0, _dt(h),
+         lim, 1.0, 0.0, None, 0)
+    return out
+
+
+_head_orders: dict = {}
+
+
+def head_project(x: torch.Tensor, w: torch.Tensor, gate: torch.Tensor | None = None) -> torch.Tensor:
+    """One small matrix per head: x [T, H * K] (head h's K columns side by side), ``w`` [H, N, K] -> out [T, H * N] with
+    out[t, h] = w[h] x[t, h]; with ``gate`` [T, H * N] (logits; rows may be a column slice of a wider tensor) the
+    result is multiplied element by element by sigmoid(gate).  Runs as the experts' grouped GEMM with the heads as
+    experts: row (t, h) belongs to "expert" h."""
+    T = x.shape[0]
+    H, N, K = w.shape
+    if not x.is_cuda:
+        o = torch.einsum("thk,hnk->thn", x.float().view(T, H, K), w.float()).reshape(T, H * N)
+        if gate is not None:
+            o = o * torch.sigmoid(gate.float())
+        return o.to(x.dtype)
+    assert x.is_contiguous() and x.shape[1] == H * K and w.is_contiguous() and w.dtype == x.dtype
+    assert gate is None or (gate.dtype == x.dtype and gate.stride(1) == 1 and gate.shape == (T, H * N)
+                            and gate.stride(0) % N == 0)
+    key = (T, H, str(x.device))
+    oo = _head_orders.get(key)
+    if oo is None:  # rows sorted by head: offs[h] = h T, order[h T + t] = t H + h
+        if len(_head_orders) > 64:
+            _head_orders.clear()
+        offs = (torch.arange(H + 1, dtype=torch.int32, device=x.device) * T).contiguous()
+        order = torch.arange(T * H, dtype=torch.int32, device=x.device).view(T, H).t().contiguous().view(-1)
+        oo = _head_orders[key] = (offs, order)
+    out = torch.empty(T, H * N, dtype=x.dtype, device=x.device)
+    # rows of N (out) and K (x) numbers: row t H + h of x viewed [T H, K] is head h of token t; the gate's row
+    # t H + h starts gate_ld / N rows of N further per token
+    call("grag_moe_gemm", ptr(x), K, ptr(w), ptr(oo[0]), ptr(oo[1]), T * H, H, 1, N, K, ptr(out), N, 2, _dt(x),
+         float("inf"), 1.0, 0.0, ptr(gate), 0 if gate is None else gate.stride(0))
     return out

@@ -171,15 +171,16 @@ def dyt_residual(resid: torch.Tensor, y: torch.Tensor | None = None, post=None, 
     return out
 
 
-def embed_gather_f32(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """Embedding rows as an fp32 [T, H] residual stream (table bf16 or fp32)."""
+def embed_gather_f32(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """Embedding rows as an fp32 [T, H] residual stream (table bf16 or fp32), multiplied by ``scale`` in fp32."""
     if not _on_gpu(table):
-        return table[ids.long()].float()
+        x = table[ids.long()].float()
+        return x if scale == 1.0 else x * scale
     ids = ids.to(torch.int32).contiguous()
     T, H = ids.numel(), table.shape[1]
     out = torch.empty(T, H, dtype=torch.float32, device=table.device)
     call("grag_embed_f32", ptr(ids), ptr(table), ptr(out), T, H, table.shape[0],
-         0 if table.dtype == torch.bfloat16 else 1)
+         0 if table.dtype == torch.bfloat16 else 1, float(scale))
     return out
 
 
@@ -231,12 +232,16 @@ def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
 def residual_rmsnorm(x: torch.Tensor, a: torch.Tensor | None = None, b: torch.Tensor | None = None,
                      bcoef: torch.Tensor | None = None, e: torch.Tensor | None = None,
                      ecoef: torch.Tensor | None = None, w: torch.Tensor | None = None, eps: float = 1e-6,
-                     out_dtype=torch.bfloat16, keep: bool = True, raw: torch.Tensor | None = None):
+                     out_dtype=torch.bfloat16, keep: bool = True, raw: torch.Tensor | None = None,
+                     gate: torch.Tensor | None = None, gbias: torch.Tensor | None = None, mult: float = 1.0):
     """One pass over the fp32 residual ``x`` [T, H] (updated in place) at the boundary of a layer whose sublayers
     read the same input: x <- x + (a + bcoef_t b + sum_k ecoef[t, k] e[t, k]) with every addend optional
     (``a``, ``b`` [T, H]; ``bcoef`` [T] fp32, None: 1; ``e`` [T, K, H] with ``ecoef`` [T, K] fp32), all summed in
     fp32; ``keep`` False: x is replaced by the sum instead.  ``raw`` [T, H] (a column slice of a wider buffer is
-    fine): receives x in ``out_dtype``.  With ``w`` [H] fp32 returns x / sqrt(mean(x^2) + eps) * w in ``out_dtype``."""
+    fine): receives x in ``out_dtype``.  With ``w`` [H] fp32 returns x / sqrt(mean(x^2) + eps) * w in ``out_dtype``.
+    A gated branch: with ``gate`` [T, H] (logits, rows may be a column slice of a wider tensor) and ``gbias`` [H] fp32
+    the sum of the addends is multiplied element by element by sigmoid(gate + gbias), and by ``mult``, before it
+    joins x."""
     assert x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
     T, H = x.shape
     K = 0 if e is None else e.shape[1]
@@ -250,6 +255,10 @@ def residual_rmsnorm(x: torch.Tensor, a: torch.Tensor | None = None, b: torch.Te
         if e is not None:
             f += (e.float() * ecoef.float()[:, :, None]).sum(1)
         y += f
+        if gate is not None:
+            y *= torch.sigmoid(gate.float() + (0.0 if gbias is None else gbias.float()))
+        if mult != 1.0:
+            y *= mult
         x.copy_(x + y if keep else y)
         if raw is not None:
             raw.copy_(x.to(raw.dtype))
@@ -260,8 +269,11 @@ def residual_rmsnorm(x: torch.Tensor, a: torch.Tensor | None = None, b: torch.Te
                          and ecoef.dtype == torch.float32 and ecoef.is_contiguous() and ecoef.shape == (T, K))
     assert bcoef is None or (bcoef.dtype == torch.float32 and bcoef.numel() == T)
     assert raw is None or (raw.dtype == out_dtype and raw.stride(1) == 1 and raw.shape == (T, H))
+    assert gate is None or (gate.dtype == out_dtype and gate.stride(1) == 1 and gate.shape == (T, H))
+    assert gbias is None or (gate is not None and gbias.dtype == torch.float32 and gbias.numel() == H)
     out = torch.empty(T, H, dtype=out_dtype, device=x.device) if w is not None else None
     call("grag_residual_rmsnorm", ptr(x), 1.0 if keep else 0.0, ptr(a), ptr(b), ptr(bcoef), ptr(e), ptr(ecoef), K,
          ptr(w), float(eps), ptr(out), ptr(raw), 0 if raw is None else raw.stride(0), T, H,
-         0 if out_dtype == torch.bfloat16 else 1)
+         0 if out_dtype == torch.bfloat16 else 1, ptr(gate), 0 if gate is None else gate.stride(0), ptr(gbias),
+         float(mult))
     return out

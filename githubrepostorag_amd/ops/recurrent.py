@@ -161,12 +161,13 @@ def _mingru_cpu(x, zoff, xoff, goff, bz, bx, state, m, W, out):
 
 # ---------------------------------------------------------------------------------------------- state-space mixer
 def causal_conv(proj: torch.Tensor, coff: int, w: torch.Tensor, b: torch.Tensor | None, cstate: torch.Tensor,
-                meta: AttnMetadata) -> torch.Tensor:
+                meta: AttnMetadata, act: bool = True, residual: bool = False) -> torch.Tensor:
     """Causal depthwise convolution + SiLU over columns coff .. coff + C of the fused projection ``proj`` [T, ld]:
     out[t, c] = silu(b[c] + sum_j w[c, j] in[t - (taps - 1) + j, c]) with ``w`` [C, taps] fp32 (the last tap is the
     current token's).  Inputs before a portion come from ``cstate`` [slots, taps - 1, C] (the sequence's last
     taps - 1 inputs, oldest first; zeros for a sequence that starts at position 0), which is brought up to date
-    after the step.  Returns [T, C] in proj's dtype."""
+    after the step.  ``act`` False: no SiLU; ``residual``: the token's own input is added to the result
+    (in + conv(in)).  Returns [T, C] in proj's dtype."""
     T = proj.shape[0]
     C, taps = w.shape
     out = torch.empty(T, C, dtype=proj.dtype, device=proj.device)
@@ -174,17 +175,17 @@ def causal_conv(proj: torch.Tensor, coff: int, w: torch.Tensor, b: torch.Tensor 
         if r1 <= r0:
             continue
         if not proj.is_cuda:
-            _causal_conv_cpu(proj[r0:r1], coff, w, b, cstate, m, out[r0:r1])
+            _causal_conv_cpu(proj[r0:r1], coff, w, b, cstate, m, out[r0:r1], act, residual)
             continue
         assert proj.stride(1) == 1 and cstate.dtype == proj.dtype and cstate.is_contiguous() and w.is_contiguous()
         assert w.dtype == torch.float32 and cstate.shape[1:] == (taps - 1, C) and taps <= lib().grag_conv_max_taps()
         call("grag_causal_conv", ptr(proj[r0:r1]), proj.stride(0), coff, C, taps, ptr(w), ptr(b), ptr(cstate),
              ptr(m.state_slots), ptr(m.q_start), ptr(m.ctx_len), ptr(out[r0:r1]), m.num_seqs, m.max_q_len,
-             cstate.shape[0], _dt(proj))
+             cstate.shape[0], _dt(proj), (0 if act else 1) | (2 if residual else 0))
     return out
 
 
-def _causal_conv_cpu(x, coff, w, b, cstate, m, out):
+def _causal_conv_cpu(x, coff, w, b, cstate, m, out, act=True, residual=False):
     C, taps = w.shape
     qs, cl, sl = m.q_start.tolist(), m.ctx_len.tolist(), m.state_slots.tolist()
     for s in range(m.num_seqs):
@@ -196,7 +197,11 @@ def _causal_conv_cpu(x, coff, w, b, cstate, m, out):
         acc = torch.zeros(e - a, C) if b is None else b.float().expand(e - a, C).clone()
         for j in range(taps):
             acc += w[:, j].float() * full[j:j + (e - a)]
-        out[a:e] = torch.nn.functional.silu(acc).to(out.dtype)
+        if act:
+            acc = torch.nn.functional.silu(acc)
+        if residual:
+            acc = acc + full[taps - 1:]
+        out[a:e] = acc.to(out.dtype)
         if taps > 1:
             cstate[sl[s]] = full[-(taps - 1):].to(cstate.dtype)
 
