@@ -290,6 +290,69 @@ latent_store_kernel(const T* __restrict__ ckv, int ld_c, const float* __restrict
   }
 }
 
+// The same out of one fused projection, for layers whose queries come straight from the layer input.  proj [T, ld]: H
+// query heads of R + r columns at column qoff, copied to q [T, H, R + r] with the last r columns of every head rotated;
+// at column coff (coff < 0: nothing is stored, the layer attends to another layer's cache) a latent of R columns and
+// the r columns of the shared key part, stored as above.  il != 0: pair i is (2i, 2i + 1) instead of (i, i + r/2).
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_rope_store_kernel(const T* __restrict__ proj, int ld, int qoff, int coff, const float* __restrict__ cw,
+                         const int* __restrict__ positions, const float* __restrict__ table, int table_rows,
+                         const int* __restrict__ slot_mapping, T* __restrict__ q, T* __restrict__ k_cache, int H, int R,
+                         int r, int BS, long nslots, float eps, int il) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63;
+  const int u = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (u > H) return;
+  int p = positions[t];
+  if (!index_ok(p, table_rows, ERR_ROPE_POS)) p = 0;
+  const float* cs = table + (size_t)p * r;
+  const int half = r >> 1;
+  if (u > 0) {
+    const T* src = proj + (size_t)t * ld + qoff + (size_t)(u - 1) * (R + r);
+    T* dst = q + ((size_t)t * H + (u - 1)) * (R + r);
+    for (int i = lane; i < R; i += 64) dst[i] = src[i];
+    for (int i = lane; i < half; i += 64) {
+      const int ia = il ? 2 * i : i, ib = il ? 2 * i + 1 : i + half;
+      const float a = ldg(src + R + ia), b = ldg(src + R + ib);
+      const float c = cs[i], s = cs[half + i];
+      stg(dst + R + ia, a * c - b * s);
+      stg(dst + R + ib, b * c + a * s);
+    }
+    return;
+  }
+  if (coff < 0) return;
+  const long slot = slot_mapping[t];
+  if (slot < 0) return;
+  if (!index_ok(slot, nslots, ERR_KV_SLOT)) return;
+  const T* src = proj + (size_t)t * ld + coff;
+  float ss = 0.f;
+  for (int i = lane; i < R; i += 64) {
+    const float v = ldg(src + i);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float rn = 1.f / sqrtf(ss / (float)R + eps);
+  T* kd = k_cache + (size_t)slot * (R + r);
+  for (int i = lane; i < R; i += 64) stg(kd + i, ldg(src + i) * rn * cw[i]);
+  for (int i = lane; i < half; i += 64) {
+    const int ia = il ? 2 * i : i, ib = il ? 2 * i + 1 : i + half;
+    const float a = ldg(src + R + ia), b = ldg(src + R + ib);
+    const float c = cs[i], s = cs[half + i];
+    stg(kd + R + ia, a * c - b * s);
+    stg(kd + R + ib, b * c + a * s);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ tanh cap
+// x [rows][ld], N columns, in place: x <- cap * tanh(x / cap) in fp32.  grid (ceil(N / 256), rows).
+template <typename T>
+__global__ void tanh_cap_kernel(T* __restrict__ x, int ld, int N, float cap, float inv) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  T* p = x + (size_t)blockIdx.y * ld + i;
+  stg(p, cap * tanhf(ldg(p) * inv));
+}
+
 // ------------------------------------------------------------------------------------------------ sigmoid window attention
 // o_i = sum over keys j with 0 <= i - j < window of sigmoid(q_i . k_j * scale + bias_h) v_j: every visible key has its
 // own weight, nothing is normalised over the keys.  K and V caches [nblk, G, BS, d | vd]; q [T, H, d]; bias [H] fp32.
@@ -692,6 +755,26 @@ GRAG_API hipError_t grag_latent_store(const void* ckv, int ld_c, const float* cw
   DT_DISPATCH(dt, hipLaunchKernelGGL(latent_store_kernel<T>, dim3(T_, (H + 4) / 4), dim3(256), 0, st, (const T*)ckv,
                                      ld_c, cw, positions, table, table_rows, slot_mapping, (T*)q, (T*)k_cache,
                                      H, R, r, BS, nslots, eps);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_latent_rope_store(const void* proj, int ld, int qoff, int coff, const float* cw,
+                                           const int* positions, const float* table, int table_rows,
+                                           const int* slot_mapping, void* q, void* k_cache, int T_, int H, int R, int r,
+                                           int BS, long nslots, float eps, int dt, int il, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  if (H + 1 > 4 * 65535 || (r & 1) || R <= 0 || (coff >= 0 && cw == nullptr)) return hipErrorInvalidValue;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(latent_rope_store_kernel<T>, dim3(T_, (H + 4) / 4), dim3(256), 0, st,
+                                     (const T*)proj, ld, qoff, coff, cw, positions, table, table_rows, slot_mapping,
+                                     (T*)q, (T*)k_cache, H, R, r, BS, nslots, eps, il);)
+  return hipGetLastError();
+}
+
+GRAG_API hipError_t grag_tanh_cap(void* x, int ld, int rows, int N, float cap, int dt, hipStream_t st) {
+  if (rows <= 0 || N <= 0) return hipSuccess;
+  if (!(cap > 0.f) || rows > 65535) return hipErrorInvalidValue;
+  DT_DISPATCH(dt, hipLaunchKernelGGL(tanh_cap_kernel<T>, dim3((N + 255) / 256, rows), dim3(256), 0, st, (T*)x, ld, N,
+                                     cap, 1.f / cap);)
   return hipGetLastError();
 }
 

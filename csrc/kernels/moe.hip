@@ -251,7 +251,47 @@ moe_align_kernel(const int* __restrict__ ids, int n, int E, int* __restrict__ of
   }
 }
 
+// ------------------------------------------------------------------------------------------------ table routing
+// ids [T][top] <- table [vocab][top] row of every token id, wts [T][top] <- 1 / top.  One thread per (token, choice).
+__global__ void moe_table_route_kernel(const int* __restrict__ tok, const int* __restrict__ table, int vocab, int top,
+                                       int* __restrict__ ids, float* __restrict__ wts, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int t = i / top, k = i - t * top;
+  const int id = tok[t];
+  ids[i] = index_ok(id, vocab, ERR_EMBED_TOKEN) ? table[(size_t)id * top + k] : -1;  // (-1: the pair is skipped)
+  wts[i] = 1.f / (float)top;
+}
+
 // ------------------------------------------------------------------------------------------------ grouped GEMM
+// The epilogue's constants.  GATED 1: the unit is g sigmoid(alpha g) (u + shift) with g = min(gate, limit),
+// u = clamp(up, -limit, limit) (limit inf, alpha 1, shift 0: SiLU(gate) * up).  GATED 2 (one matrix per attention head:
+// the "experts" are the E heads, `top` holds the token count, row r of the sorted order is token r % top of head
+// r / top, i.e. row (r % top) * E + r / top of a and out -- no offs / order arrays): with `gate`, element (t, h, n) of
+// the result is multiplied by sigmoid(gate[t * gate_ld + h * N + n]).
+struct MoeEpi {
+  float limit, alpha, shift;
+  const void* gate;
+  int gate_ld;
+};
+__device__ __forceinline__ float glu_unit(float g, float u, const MoeEpi& ep) {
+  g = fminf(g, ep.limit);
+  u = fminf(fmaxf(u, -ep.limit), ep.limit);
+  return g / (1.f + expf(-ep.alpha * g)) * (u + ep.shift);
+}
+template <int GATED> __device__ __forceinline__ int moe_off(const int* offs, int e, int top) {
+  return GATED == 2 ? e * top : offs[e];
+}
+template <int GATED> __device__ __forceinline__ int moe_order(const int* order, int r, int top, int E) {
+  return GATED == 2 ? (r % top) * E + r / top : order[r];
+}
+template <int GATED, typename T>
+__device__ __forceinline__ float head_gate_of(const MoeEpi& ep, size_t orow, int n, int E, int N) {
+  if (GATED != 2 || ep.gate == nullptr) return 1.f;
+  const size_t t = orow / E, h = orow - t * E;
+  const float z = (float)reinterpret_cast<const T*>(ep.gate)[t * ep.gate_ld + h * N + n];
+  return 1.f / (1.f + expf(-z));
+}
 // Rows sorted by expert; the workgroup of row tile blockIdx.y finds its expert by walking offs (tiles never straddle
 // two experts).  GATED 1: A row r = h[order[r] / top] (gathered), B = wgu[e] ([2F][K]: gate rows, then up rows),
 // out[r][n] = silu(a . gate_n) * (a . up_n), out [rows][F] in sorted order.  GATED 0: A row r = act[r] (sorted order),
@@ -263,14 +303,14 @@ constexpr int MG_M = 32, MG_N = 64, MG_K = 32;
 template <typename T, int GATED>
 __global__ void __launch_bounds__(256)
 moe_gemm_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, const int* __restrict__ offs,
-                const int* __restrict__ order, int E, int top, int N, int K, T* __restrict__ out, int ldo) {
+                const int* __restrict__ order, int E, int top, int N, int K, T* __restrict__ out, int ldo, MoeEpi ep) {
   __shared__ float As[MG_M][MG_K + 1];
-  __shared__ float Bs[GATED ? 2 : 1][MG_N][MG_K + 1];
+  __shared__ float Bs[GATED == 1 ? 2 : 1][MG_N][MG_K + 1];
   __shared__ int rows[MG_M];
   // the expert and row range of this tile
   int e = 0, tile = blockIdx.y, r0 = -1, rend = 0;
   for (; e < E; ++e) {
-    const int b = offs[e], n = offs[e + 1] - b, nt = (n + MG_M - 1) / MG_M;
+    const int b = moe_off<GATED>(offs, e, top), n = moe_off<GATED>(offs, e + 1, top) - b, nt = (n + MG_M - 1) / MG_M;
     if (tile < nt) {
       r0 = b + tile * MG_M;
       rend = b + n;
@@ -283,13 +323,13 @@ moe_gemm_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, const
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
   if (threadIdx.x < MG_M) {
     const int r = r0 + threadIdx.x;
-    rows[threadIdx.x] = r < rend ? (GATED ? order[r] / top : r) : -1;
+    rows[threadIdx.x] = r < rend ? (GATED == 1 ? order[r] / top : GATED == 2 ? moe_order<2>(order, r, top, E) : r) : -1;
   }
-  const size_t wrows = GATED ? (size_t)2 * N : (size_t)N;
+  const size_t wrows = GATED == 1 ? (size_t)2 * N : (size_t)N;
   const T* we = w + (size_t)e * wrows * K;
-  float acc[GATED ? 2 : 1][2][4];
+  float acc[GATED == 1 ? 2 : 1][2][4];
 #pragma unroll
-  for (int u = 0; u < (GATED ? 2 : 1); ++u)
+  for (int u = 0; u < (GATED == 1 ? 2 : 1); ++u)
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -305,14 +345,14 @@ moe_gemm_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, const
       const int n = idx / MG_K, k = idx - n * MG_K;
       const bool ok = n0 + n < N && k0 + k < K;
       Bs[0][n][k] = ok ? ldm(we + (size_t)(n0 + n) * K + k0 + k) : 0.f;
-      if (GATED) Bs[GATED ? 1 : 0][n][k] = ok ? ldm(we + (size_t)(N + n0 + n) * K + k0 + k) : 0.f;
+      if (GATED == 1) Bs[GATED == 1 ? 1 : 0][n][k] = ok ? ldm(we + (size_t)(N + n0 + n) * K + k0 + k) : 0.f;
     }
     __syncthreads();
 #pragma unroll 8
     for (int k = 0; k < MG_K; ++k) {
       const float a0 = As[ty][k], a1 = As[ty + 16][k];
 #pragma unroll
-      for (int u = 0; u < (GATED ? 2 : 1); ++u)
+      for (int u = 0; u < (GATED == 1 ? 2 : 1); ++u)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float b = Bs[u][tx + 16 * j][k];
@@ -325,13 +365,14 @@ moe_gemm_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, const
   for (int i = 0; i < 2; ++i) {
     const int r = r0 + ty + 16 * i;
     if (r >= rend) continue;
-    const size_t orow = GATED ? (size_t)r : (size_t)order[r];
+    const size_t orow = GATED == 1 ? (size_t)r : (size_t)moe_order<GATED>(order, r, top, E);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx + 16 * j;
       if (n >= N) continue;
       float v = acc[0][i][j];
-      if (GATED) v = v / (1.f + expf(-v)) * acc[GATED ? 1 : 0][i][j];
+      if (GATED == 1) v = glu_unit(v, acc[GATED == 1 ? 1 : 0][i][j], ep);
+      if (GATED == 2) v *= head_gate_of<GATED, T>(ep, orow, n, E, N);
       stm(out + orow * ldo + n, v);
     }
   }
@@ -344,14 +385,14 @@ moe_gemm_kernel(const T* __restrict__ a, int lda, const T* __restrict__ w, const
 template <int GATED>
 __global__ void __launch_bounds__(256)
 moe_gemm_mfma_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, const int* __restrict__ offs,
-                     const int* __restrict__ order, int E, int top, int N, int K, bf16* __restrict__ out, int ldo) {
+                     const int* __restrict__ order, int E, int top, int N, int K, bf16* __restrict__ out, int ldo, MoeEpi ep) {
   constexpr int KS = MG_K + 8;  // LDS row stride (elements): 80 bytes, 16-byte aligned rows
   __shared__ __attribute__((aligned(16))) short As[MG_M][KS];
-  __shared__ __attribute__((aligned(16))) short Bs[GATED ? 2 : 1][MG_N][KS];
+  __shared__ __attribute__((aligned(16))) short Bs[GATED == 1 ? 2 : 1][MG_N][KS];
   __shared__ int rows[MG_M];
   int e = 0, tile = blockIdx.y, r0 = -1, rend = 0;
   for (; e < E; ++e) {
-    const int b = offs[e], n = offs[e + 1] - b, nt = (n + MG_M - 1) / MG_M;
+    const int b = moe_off<GATED>(offs, e, top), n = moe_off<GATED>(offs, e + 1, top) - b, nt = (n + MG_M - 1) / MG_M;
     if (tile < nt) {
       r0 = b + tile * MG_M;
       rend = b + n;
@@ -366,13 +407,13 @@ moe_gemm_mfma_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict
   const int wr = (wid >> 1) * 16, wc = (wid & 1) * 32;
   if (threadIdx.x < MG_M) {
     const int r = r0 + threadIdx.x;
-    rows[threadIdx.x] = r < rend ? (GATED ? order[r] / top : r) : -1;
+    rows[threadIdx.x] = r < rend ? (GATED == 1 ? order[r] / top : GATED == 2 ? moe_order<2>(order, r, top, E) : r) : -1;
   }
-  const size_t wrows = GATED ? (size_t)2 * N : (size_t)N;
+  const size_t wrows = GATED == 1 ? (size_t)2 * N : (size_t)N;
   const bf16* we = w + (size_t)e * wrows * K;
-  f32x4_t acc[GATED ? 2 : 1][2];
+  f32x4_t acc[GATED == 1 ? 2 : 1][2];
 #pragma unroll
-  for (int u = 0; u < (GATED ? 2 : 1); ++u)
+  for (int u = 0; u < (GATED == 1 ? 2 : 1); ++u)
 #pragma unroll
     for (int c = 0; c < 2; ++c) acc[u][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   __syncthreads();
@@ -386,18 +427,18 @@ moe_gemm_mfma_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict
     }
     if (n0 + sr < N && k0 + sv < K) {
       bv0 = *reinterpret_cast<const bf16x8_t*>(we + (size_t)(n0 + sr) * K + k0 + sv);
-      if (GATED) bv1 = *reinterpret_cast<const bf16x8_t*>(we + (size_t)(N + n0 + sr) * K + k0 + sv);
+      if (GATED == 1) bv1 = *reinterpret_cast<const bf16x8_t*>(we + (size_t)(N + n0 + sr) * K + k0 + sv);
     }
     __syncthreads();
     if (threadIdx.x < 128) *reinterpret_cast<bf16x8_t*>(&As[sr][sv]) = av;
     *reinterpret_cast<bf16x8_t*>(&Bs[0][sr][sv]) = bv0;
-    if (GATED) *reinterpret_cast<bf16x8_t*>(&Bs[GATED ? 1 : 0][sr][sv]) = bv1;
+    if (GATED == 1) *reinterpret_cast<bf16x8_t*>(&Bs[GATED == 1 ? 1 : 0][sr][sv]) = bv1;
     __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < MG_K / 16; ++ks) {
       const bf16x4_t af = *reinterpret_cast<const bf16x4_t*>(&As[wr + ql][ks * 16 + quad * 4]);
 #pragma unroll
-      for (int u = 0; u < (GATED ? 2 : 1); ++u)
+      for (int u = 0; u < (GATED == 1 ? 2 : 1); ++u)
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
           const bf16x4_t bf = *reinterpret_cast<const bf16x4_t*>(&Bs[u][wc + 16 * c + ql][ks * 16 + quad * 4]);
@@ -409,13 +450,14 @@ moe_gemm_mfma_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict
   for (int i = 0; i < 4; ++i) {
     const int r = r0 + wr + 4 * quad + i;
     if (r >= rend) continue;
-    const size_t orow = GATED ? (size_t)r : (size_t)order[r];
+    const size_t orow = GATED == 1 ? (size_t)r : (size_t)moe_order<GATED>(order, r, top, E);
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
       const int n = n0 + wc + 16 * c + ql;
       if (n >= N) continue;
       float v = acc[0][c][i];
-      if (GATED) v = v / (1.f + expf(-v)) * acc[GATED ? 1 : 0][c][i];
+      if (GATED == 1) v = glu_unit(v, acc[GATED == 1 ? 1 : 0][c][i], ep);
+      if (GATED == 2) v *= head_gate_of<GATED, bf16>(ep, orow, n, E, N);
       out[orow * ldo + n] = (bf16)v;
     }
   }
@@ -428,14 +470,14 @@ moe_gemm_mfma_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict
 template <int GATED>
 __global__ void __launch_bounds__(256, 2)
 moe_gemm_big_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict__ w, const int* __restrict__ offs,
-                    const int* __restrict__ order, int E, int top, int N, int K, bf16* __restrict__ out, int ldo) {
-  constexpr int TM = 128, TN = 128, TK = 64, KS = TK + 8, NB = GATED ? 2 : 1;
+                    const int* __restrict__ order, int E, int top, int N, int K, bf16* __restrict__ out, int ldo, MoeEpi ep) {
+  constexpr int TM = 128, TN = 128, TK = 64, KS = TK + 8, NB = GATED == 1 ? 2 : 1;
   __shared__ __attribute__((aligned(16))) short As[TM][KS];
   __shared__ __attribute__((aligned(16))) short Bs[NB][TN][KS];
   __shared__ int rows[TM];
   int e = 0, tile = blockIdx.y, r0 = -1, rend = 0;
   for (; e < E; ++e) {
-    const int b = offs[e], n = offs[e + 1] - b, nt = (n + TM - 1) / TM;
+    const int b = moe_off<GATED>(offs, e, top), n = moe_off<GATED>(offs, e + 1, top) - b, nt = (n + TM - 1) / TM;
     if (tile < nt) {
       r0 = b + tile * TM;
       rend = b + n;
@@ -450,10 +492,10 @@ moe_gemm_big_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict_
   const int wr = (wid >> 1) * 64, wc = (wid & 1) * 64;
   if (threadIdx.x < TM) {
     const int r = r0 + threadIdx.x;
-    rows[threadIdx.x] = r < rend ? (GATED ? order[r] / top : r) : -1;
+    rows[threadIdx.x] = r < rend ? (GATED == 1 ? order[r] / top : GATED == 2 ? moe_order<2>(order, r, top, E) : r) : -1;
   }
   __syncthreads();
-  const size_t wrows = GATED ? (size_t)2 * N : (size_t)N;
+  const size_t wrows = GATED == 1 ? (size_t)2 * N : (size_t)N;
   const bf16* we = w + (size_t)e * wrows * K;
   // staging: thread t owns rows t / 8 + 32 u (u < 4) of every tile, 16-byte vector (t % 8) of the K step
   constexpr int NU = 4;
@@ -521,20 +563,22 @@ moe_gemm_big_kernel(const bf16* __restrict__ a, int lda, const bf16* __restrict_
     for (int c = 0; c < 4; ++c) {
       const int r = r0 + wr + 16 * i + 4 * quad + c;
       if (r >= rend) continue;
-      const size_t orow = GATED ? (size_t)r : (size_t)order[r];
+      const size_t orow = GATED == 1 ? (size_t)r : (size_t)moe_order<GATED>(order, r, top, E);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int n = n0 + wc + 16 * j + ql;
         if (n >= N) continue;
         float v = acc[0][i][j][c];
-        if (GATED) v = v / (1.f + expf(-v)) * acc[NB - 1][i][j][c];
+        if (GATED == 1) v = glu_unit(v, acc[NB - 1][i][j][c], ep);
+        if (GATED == 2) v *= head_gate_of<GATED, bf16>(ep, orow, n, E, N);
         out[orow * ldo + n] = (bf16)v;
       }
     }
 }
 
 // ------------------------------------------------------------------------------------------------ residual boundary
-// x [T][H] fp32, in place: x <- keep x + (a + bcoef_t b + sum_k ecoef_(t,k) e_(t,k)), every addend optional
+// x [T][H] fp32, in place: x <- keep x + mult * sigmoid(gate + gbias) * (a + bcoef_t b + sum_k ecoef_(t,k) e_(t,k)), every
+// addend optional, the gate too (gate [T][gate_ld] logits in the activation type, gbias [H] fp32)
 // (a, b [T][H]; e [T * K][H], ecoef [T * K]; bcoef [T], null: 1).  Then, each optional: raw [T][raw_ld] <- x in the
 // activation type, out [T][H] <- x / sqrt(mean(x^2) + eps) * w.  grid (T), 256 threads; a thread keeps its elements of
 // the row in registers between the sum of squares and the scaling (rows of up to 256 * RB_PER), or re-reads x.
@@ -545,7 +589,8 @@ __global__ void __launch_bounds__(256)
 residual_rmsnorm_kernel(float* __restrict__ x, float keep, const T* __restrict__ a, const T* __restrict__ b,
                         const float* __restrict__ bcoef, const T* __restrict__ e, const float* __restrict__ ecoef,
                         int K, const float* __restrict__ w, float eps, T* __restrict__ out, T* __restrict__ raw,
-                        int raw_ld, int H) {
+                        int raw_ld, int H, const T* __restrict__ gate, int gate_ld, const float* __restrict__ gbias,
+                        float mult) {
   __shared__ float red[16];
   const size_t t = blockIdx.x, row = t * H;
   const float bc = b ? (bcoef ? bcoef[t] : 1.f) : 0.f;
@@ -562,6 +607,8 @@ residual_rmsnorm_kernel(float* __restrict__ x, float keep, const T* __restrict__
       float f = b ? bc * ldm(b + row + i) : 0.f;
       for (int k = 0; k < K; ++k) f = fmaf(ecoef[t * K + k], ldm(e + (t * K + k) * H + i), f);
       y += f;
+      if (gate) y *= 1.f / (1.f + expf(-(ldm(gate + t * gate_ld + i) + (gbias ? gbias[i] : 0.f))));
+      y *= mult;
       const float nx = keep != 0.f ? keep * x[row + i] + y : y;
       x[row + i] = nx;
       v[u] = nx;
@@ -575,6 +622,8 @@ residual_rmsnorm_kernel(float* __restrict__ x, float keep, const T* __restrict__
       float f = b ? bc * ldm(b + row + i) : 0.f;
       for (int k = 0; k < K; ++k) f = fmaf(ecoef[t * K + k], ldm(e + (t * K + k) * H + i), f);
       y += f;
+      if (gate) y *= 1.f / (1.f + expf(-(ldm(gate + t * gate_ld + i) + (gbias ? gbias[i] : 0.f))));
+      y *= mult;
       const float nx = keep != 0.f ? keep * x[row + i] + y : y;
       x[row + i] = nx;
       ss = fmaf(nx, nx, ss);
@@ -615,7 +664,8 @@ __global__ void __launch_bounds__(256)
 residual_rmsnorm_vec_kernel(float* __restrict__ x, float keep, const T* __restrict__ a, const T* __restrict__ b,
                             const float* __restrict__ bcoef, const T* __restrict__ e, const float* __restrict__ ecoef,
                             int K, const float* __restrict__ w, float eps, T* __restrict__ out, T* __restrict__ raw,
-                            int raw_ld, int H) {
+                            int raw_ld, int H, const T* __restrict__ gate, int gate_ld,
+                            const float* __restrict__ gbias, float mult) {
   __shared__ float red[16];
   const size_t t = blockIdx.x, row = t * H;
   const float bc = b ? (bcoef ? bcoef[t] : 1.f) : 0.f;
@@ -635,6 +685,13 @@ residual_rmsnorm_vec_kernel(float* __restrict__ x, float keep, const T* __restri
         for (int r = 0; r < 4; ++r) f[r] = fmaf(c, ev[r], f[r]);
       }
       y += f;
+      if (gate) {
+        const f32x4_t gv = ld4(gate + t * gate_ld + i);
+        const f32x4_t gb = gbias ? *reinterpret_cast<const f32x4_t*>(gbias + i) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) y[r] *= 1.f / (1.f + expf(-(gv[r] + gb[r])));
+      }
+      y *= mult;
       f32x4_t nx = y;
       if (keep != 0.f) {
         const f32x4_t xv = *reinterpret_cast<const f32x4_t*>(x + row + i);
@@ -710,63 +767,81 @@ GRAG_API hipError_t grag_moe_align(const int* ids, int n, int E, int* offs, int*
   return hipGetLastError();
 }
 
+GRAG_API hipError_t grag_moe_table_route(const int* tok, const int* table, int vocab, int top, int* ids, float* wts,
+                                         int T_, hipStream_t st) {
+  if (T_ <= 0) return hipSuccess;
+  if (top < 1 || vocab < 1) return hipErrorInvalidValue;
+  const int n = T_ * top;
+  hipLaunchKernelGGL(moe_table_route_kernel, dim3((n + 255) / 256), dim3(256), 0, st, tok, table, vocab, top, ids, wts, n);
+  return hipGetLastError();
+}
+
 // rows = T * top sorted rows.  gated 1: a = h [T][lda], w = [E][2N][K], out [rows][N]; gated 0: a = [rows][lda] sorted,
-// w = [E][N][K], out [rows][ldo] in (token, choice) order.
+// w = [E][N][K], out [rows][ldo] in (token, choice) order; gated 2: one matrix per head (E heads, top = tokens, rows =
+// tokens * E): a = [tokens * E][lda], w = [E][N][K], out [tokens * E][ldo], offs / order unused.
 GRAG_API hipError_t grag_moe_gemm(const void* a, int lda, const void* w, const int* offs, const int* order, int rows,
-                                  int E, int top, int N, int K, void* out, int ldo, int gated, int dt, hipStream_t st) {
+                                  int E, int top, int N, int K, void* out, int ldo, int gated, int dt, float limit,
+                                  float alpha, float shift, const void* gate, int gate_ld, hipStream_t st) {
   if (rows <= 0) return hipSuccess;
   const int tiles = (rows + MG_M - 1) / MG_M + E;  // every expert may end on a partial tile
-  if (tiles > 65535 || E < 1 || top < 1) return hipErrorInvalidValue;
+  if (tiles > 65535 || E < 1 || top < 1 || gated < 0 || gated > 2) return hipErrorInvalidValue;
+  if (gated == 2 ? rows != E * top : (offs == nullptr || order == nullptr)) return hipErrorInvalidValue;
+  const MoeEpi ep{limit, alpha, shift, gate, gate_ld};
   const dim3 grid((N + MG_N - 1) / MG_N, tiles);
   auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+#define MOE_LAUNCH(KERN, GRID, A, W, O)                                                                             \
+  {                                                                                                                  \
+    if (gated == 1)                                                                                                  \
+      hipLaunchKernelGGL((KERN<1>), GRID, dim3(256), 0, st, A, lda, W, offs, order, E, top, N, K, O, ldo, ep);       \
+    else if (gated == 2)                                                                                             \
+      hipLaunchKernelGGL((KERN<2>), GRID, dim3(256), 0, st, A, lda, W, offs, order, E, top, N, K, O, ldo, ep);       \
+    else                                                                                                             \
+      hipLaunchKernelGGL((KERN<0>), GRID, dim3(256), 0, st, A, lda, W, offs, order, E, top, N, K, O, ldo, ep);       \
+  }
   if (dt == 0 && K % 8 == 0 && lda % 8 == 0 && al16(a) && al16(w) && rows >= 48 * E) {
     // prompt-sized row counts (half a large tile per expert on average, or more): the 128 x 128 tiles
     const int btiles = (rows + 127) / 128 + E;
     const dim3 bgrid((N + 127) / 128, btiles);
-    if (gated)
-      hipLaunchKernelGGL(moe_gemm_big_kernel<1>, bgrid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,
-                         order, E, top, N, K, (bf16*)out, ldo);
-    else
-      hipLaunchKernelGGL(moe_gemm_big_kernel<0>, bgrid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,
-                         order, E, top, N, K, (bf16*)out, ldo);
+    MOE_LAUNCH(moe_gemm_big_kernel, bgrid, (const bf16*)a, (const bf16*)w, (bf16*)out)
     return hipGetLastError();
   }
   if (dt == 0 && K % 8 == 0 && lda % 8 == 0 && al16(a) && al16(w)) {
-    if (gated)
-      hipLaunchKernelGGL(moe_gemm_mfma_kernel<1>, grid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,
-                         order, E, top, N, K, (bf16*)out, ldo);
-    else
-      hipLaunchKernelGGL(moe_gemm_mfma_kernel<0>, grid, dim3(256), 0, st, (const bf16*)a, lda, (const bf16*)w, offs,
-                         order, E, top, N, K, (bf16*)out, ldo);
+    MOE_LAUNCH(moe_gemm_mfma_kernel, grid, (const bf16*)a, (const bf16*)w, (bf16*)out)
     return hipGetLastError();
   }
+#undef MOE_LAUNCH
   DT_DISPATCH(dt, {
-    if (gated)
+    if (gated == 1)
       hipLaunchKernelGGL((moe_gemm_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)a, lda, (const T*)w, offs, order, E,
-                         top, N, K, (T*)out, ldo);
+                         top, N, K, (T*)out, ldo, ep);
+    else if (gated == 2)
+      hipLaunchKernelGGL((moe_gemm_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)a, lda, (const T*)w, offs, order, E,
+                         top, N, K, (T*)out, ldo, ep);
     else
       hipLaunchKernelGGL((moe_gemm_kernel<T, 0>), grid, dim3(256), 0, st, (const T*)a, lda, (const T*)w, offs, order, E,
-                         top, N, K, (T*)out, ldo);
+                         top, N, K, (T*)out, ldo, ep);
   })
   return hipGetLastError();
 }
 
 GRAG_API hipError_t grag_residual_rmsnorm(float* x, float keep, const void* a, const void* b, const float* bcoef,
                                           const void* e, const float* ecoef, int K, const float* w, float eps,
-                                          void* out, void* raw, int raw_ld, int T_, int H, int dt, hipStream_t st) {
+                                          void* out, void* raw, int raw_ld, int T_, int H, int dt, const void* gate,
+                                          int gate_ld, const float* gbias, float mult, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
-  if (K < 0 || (K > 0 && (e == nullptr || ecoef == nullptr)) || (out != nullptr && w == nullptr))
+  if (K < 0 || (K > 0 && (e == nullptr || ecoef == nullptr)) || (out != nullptr && w == nullptr) ||
+      (gbias != nullptr && gate == nullptr))
     return hipErrorInvalidValue;
   auto al16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   if (H % 4 == 0 && H <= 4 * 256 * RBV_PER && al16(x) && al16(a) && al16(b) && al16(e) && al16(w) && al16(out) &&
-      al16(raw) && raw_ld % 8 == 0) {
+      al16(raw) && raw_ld % 8 == 0 && al16(gate) && al16(gbias) && gate_ld % 8 == 0) {
     DT_DISPATCH(dt, hipLaunchKernelGGL(residual_rmsnorm_vec_kernel<T>, dim3(T_), dim3(256), 0, st, x, keep,
                                        (const T*)a, (const T*)b, bcoef, (const T*)e, ecoef, e ? K : 0, w, eps, (T*)out,
-                                       (T*)raw, raw_ld, H);)
+                                       (T*)raw, raw_ld, H, (const T*)gate, gate_ld, gbias, mult);)
     return hipGetLastError();
   }
   DT_DISPATCH(dt, hipLaunchKernelGGL(residual_rmsnorm_kernel<T>, dim3(T_), dim3(256), 0, st, x, keep, (const T*)a,
                                      (const T*)b, bcoef, (const T*)e, ecoef, e ? K : 0, w, eps, (T*)out, (T*)raw,
-                                     raw_ld, H);)
+                                     raw_ld, H, (const T*)gate, gate_ld, gbias, mult);)
   return hipGetLastError();
 }

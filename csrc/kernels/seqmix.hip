@@ -38,7 +38,7 @@ __device__ __forceinline__ float tanh_acc(float x) {
 // ------------------------------------------------------------------------------------------------ embedding
 template <typename T>
 __global__ void embed_f32_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
-                                 int H, int vocab) {
+                                 int H, int vocab, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   if (!index_ok(id, vocab, ERR_EMBED_TOKEN)) {
@@ -46,7 +46,7 @@ __global__ void embed_f32_kernel(const int* __restrict__ ids, const T* __restric
     return;
   }
   const T* row = table + (size_t)id * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) out[(size_t)t * H + i] = ldf(row + i);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[(size_t)t * H + i] = ldf(row + i) * scale;
 }
 
 // ------------------------------------------------------------------------------------------------ Dynamic Tanh
@@ -165,19 +165,28 @@ __global__ void rope_vnorm_store_kernel(const T* __restrict__ proj, int ld, int 
 // Optional extras (AttnExtra, all off when zero): `hscale` [H] multiplies the score scale of head h (a temperature per
 // head); `chunk` > 0 confines a query at position i to the keys j of its own aligned block of `chunk` positions,
 // floor(j / chunk) == floor(i / chunk) (and j <= i); `hgate` [T][gate_ld] holds one logit per (token, head) and the
-// head's output is multiplied by its sigmoid as it is stored.
+// head's output is multiplied by its sigmoid as it is stored; `window` > 0 is sliding-window attention, a query at
+// position i sees key j only when 0 <= i - j < window; `softcap` > 0 sends every scaled score s through
+// softcap * tanh(s / softcap) before the softmax.
 struct AttnExtra {
   const float* hscale;
   const void* hgate;
   int gate_ld;
   int chunk;
+  int window;
+  float softcap;
 };
 template <typename T>
 __device__ __forceinline__ float head_gate(const AttnExtra& ex, size_t row, int h) {
   return ex.hgate ? sigmoid_acc(ldf(reinterpret_cast<const T*>(ex.hgate) + row * ex.gate_ld + h)) : 1.f;
 }
+// the first key the query at position `pos` sees (never falls as pos grows)
 __device__ __forceinline__ int chunk_start(const AttnExtra& ex, int pos) {
-  return ex.chunk > 0 ? pos - pos % ex.chunk : 0;
+  const int lo = ex.chunk > 0 ? pos - pos % ex.chunk : 0;
+  return ex.window > 0 ? max(lo, pos - ex.window + 1) : lo;
+}
+__device__ __forceinline__ float cap_score(const AttnExtra& ex, float s) {
+  return ex.softcap > 0.f ? ex.softcap * tanhf(s / ex.softcap) : s;
 }
 
 constexpr int SA_NQ = 4;   // queries per wave (prefill)
@@ -262,7 +271,7 @@ sink_attn_prefill_kernel(const T* __restrict__ q, const T* __restrict__ k_cache,
     for (int n = 0; n < SA_NQ; ++n) {
       const int tq = q0 + wid * SA_NQ + n;
       const bool vis = lane < kn && tq < qlen && (k0 + lane) <= pos0 + tq && (k0 + lane) >= chunk_start(ex, pos0 + tq);
-      const float sc = vis ? s[n] * scale : -INFINITY;
+      const float sc = vis ? cap_score(ex, s[n] * scale) : -INFINITY;
       const float mn = fmaxf(m[n], wave_max(sc));
       const float p = vis ? expf(sc - mn) : 0.f;
       const float alpha = expf(m[n] - mn);
@@ -402,6 +411,13 @@ sink_attn_prefill_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict
     // a tile wholly at or before the wave's first query (and inside the context) needs no mask
     const bool interior = k0 + KT - 1 <= pos0 + q0 + wid * 16 && k0 + KT <= nkeys && q0 + wid * 16 + 15 < qlen &&
                           k0 >= wave_cmax;
+    if (ex.softcap > 0.f) {  // cap in the natural domain, then to log2
+      const float s1 = scale * (ex.hscale ? ex.hscale[h] : 1.f), ic = 1.f / ex.softcap, c2 = ex.softcap * LOG2E;
+#pragma unroll
+      for (int n = 0; n < 4; ++n)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) st[n][i] = c2 * tanhf(st[n][i] * s1 * ic) / sc2;
+    }
     if (interior) {
 #pragma unroll
       for (int n = 0; n < 4; ++n)
@@ -584,7 +600,7 @@ sink_attn_decode_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict_
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const bool vis = col_ok && 16 * wid + 4 * quad + i < kn;
-        st[i] = vis ? st[i] * scale : -INFINITY;
+        st[i] = vis ? cap_score(ex, st[i] * scale) : -INFINITY;
         tmax = fmaxf(tmax, st[i]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
@@ -746,7 +762,7 @@ sink_attn_decode_vec_kernel(const bf16* __restrict__ q, const bf16* __restrict__
         for (int e = 0; e < 8; ++e) s = fmaf(Qs[c * 8 + e], bits2f(kv[e]), s);
       }
     }
-    const float sc = vis ? s * scale : -INFINITY;
+    const float sc = vis ? cap_score(ex, s * scale) : -INFINITY;
     const float mn = fmaxf(m, wave_max(sc));
     const float p = vis ? expf(sc - mn) : 0.f;
     const float alpha = (m == -INFINITY) ? 0.f : expf(m - mn);
@@ -845,7 +861,7 @@ sink_attn_decode_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, 
       const T* kr = k_cache + (((size_t)blk * G + g) * BS + key % BS) * d;
       for (int i = 0; i < d; ++i) s = fmaf(Qs[i], ldf(kr + i), s);
     }
-    const float sc = vis ? s * scale : -INFINITY;
+    const float sc = vis ? cap_score(ex, s * scale) : -INFINITY;
     const float mn = fmaxf(m, wave_max(sc));  // (wave 0 always has the finite sink; others see >= 1 visible key)
     const float p = vis ? expf(sc - mn) : 0.f;
     const float alpha = (m == -INFINITY) ? 0.f : expf(m - mn);
@@ -1239,10 +1255,10 @@ using namespace grag;
   }
 
 GRAG_API hipError_t grag_embed_f32(const int* ids, const void* table, float* out, int T_, int H, int vocab, int dt,
-                                   hipStream_t st) {
+                                   float scale, hipStream_t st) {
   if (T_ <= 0) return hipSuccess;
   DT_DISPATCH(dt, hipLaunchKernelGGL(embed_f32_kernel<T>, dim3(T_), dim3(256), 0, st, ids, (const T*)table, out, H,
-                                     vocab);)
+                                     vocab, scale);)
   return hipGetLastError();
 }
 
@@ -1290,8 +1306,8 @@ GRAG_API hipError_t grag_sink_attn_prefill(const void* q, const void* k_cache, c
                                            const int* ctx_len, const float* sinks, int nseq, int max_q_len, int H,
                                            int G, int d, int vd, int BS, float scale, float out_scale, int nblocks,
                                            int dt, int v_ld, const float* hscale, const void* hgate, int gate_ld,
-                                           int chunk, hipStream_t st) {
-  const AttnExtra ex{hscale, hgate, gate_ld, chunk};
+                                           int chunk, int window, float softcap, hipStream_t st) {
+  const AttnExtra ex{hscale, hgate, gate_ld, chunk, window, softcap};
   // v_ld: elements from one cached value row to the next (vd, or more when the value rows are the head of wider rows)
   if (nseq <= 0 || max_q_len <= 0) return hipSuccess;
   if (vd > 64 * SA_VC || G <= 0 || H % G || v_ld < vd) return hipErrorInvalidValue;
@@ -1343,8 +1359,9 @@ GRAG_API hipError_t grag_sink_attn_decode(const void* q, const void* k_cache, co
                                           const float* sinks, int nseq, int H, int G, int d, int vd, int BS,
                                           float scale, float out_scale, int nblocks, int dt, int nsplit,
                                           int split_len, float* part_o, float* part_ml, int v_ld, const float* hscale,
-                                          const void* hgate, int gate_ld, int chunk, hipStream_t st) {
-  const AttnExtra ex{hscale, hgate, gate_ld, chunk};
+                                          const void* hgate, int gate_ld, int chunk, int window, float softcap,
+                                          hipStream_t st) {
+  const AttnExtra ex{hscale, hgate, gate_ld, chunk, window, softcap};
   if (nseq <= 0) return hipSuccess;
   if (vd > 64 * SA_VC || G <= 0 || H % G || v_ld < vd) return hipErrorInvalidValue;
   if (dt == 0 && v_ld % 8 == 0 && (reinterpret_cast<uintptr_t>(v_cache) & 15) == 0 && d % 16 == 0 && vd % 16 == 0 && d <= 256 && vd <= 256 && G * ((H / G + 15) / 16) <= 65535 &&
@@ -1417,7 +1434,7 @@ GRAG_API hipError_t grag_window_decode_mfma(const void* q, const void* k_cache, 
     hipLaunchKernelGGL((sink_attn_decode_mfma_kernel<NK, NV, 1>), mgrid, dim3(256), mb, st, (const bf16*)q,          \
                        (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, out_ld, block_tables, bt_stride,      \
                        ctx_len, bias, H, G, d, vd, BS, scale, 1.f, nblocks, 1, 0, (float*)nullptr, (float*)nullptr,  \
-                       window, (const bf16*)gate, gate_ld, vd, AttnExtra{nullptr, nullptr, 0, 0});                   \
+                       window, (const bf16*)gate, gate_ld, vd, AttnExtra{nullptr, nullptr, 0, 0, 0, 0.f});                   \
   }
   if (d <= 64 && vd <= 64) SW_MFMA(4, 4)
   else SW_MFMA(8, 8)

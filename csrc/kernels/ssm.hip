@@ -28,12 +28,14 @@ constexpr int CONV_TT = 16;  // tokens per workgroup
 
 // out [T][C] = SiLU(b[c] + sum_j w[c][j] in[t - (taps - 1) + j][c]), in = proj columns coff .. coff + C; inputs before
 // the portion come from cstate [slots][taps - 1][C] (oldest first), zeros for a sequence that starts at position 0.
+// mode bit 0: no SiLU; bit 1: the token's own input is added to the result (in + conv(in)).
 // grid (ceil(C / 256), ceil(max_q_len / CONV_TT), nseq).  The pool is only read here.
 template <typename T>
 __global__ void __launch_bounds__(256)
 causal_conv_kernel(const T* __restrict__ proj, int ld, int coff, int C, int taps, const float* __restrict__ w,
                    const float* __restrict__ b, const T* __restrict__ cstate, const int* __restrict__ slots,
-                   const int* __restrict__ q_start, const int* __restrict__ ctx_len, T* __restrict__ out, int nslots) {
+                   const int* __restrict__ q_start, const int* __restrict__ ctx_len, T* __restrict__ out, int nslots,
+                   int mode) {
   const int seq = blockIdx.z, c = blockIdx.x * 256 + threadIdx.x;
   const int qa = q_start[seq], qlen = q_start[seq + 1] - qa;
   const int t0 = blockIdx.y * CONV_TT;
@@ -65,7 +67,9 @@ causal_conv_kernel(const T* __restrict__ proj, int ld, int coff, int C, int taps
       if (j < taps - 1) acc = fmaf(wt[j], win[j], acc);
     }
     acc = fmaf(wlast, cur, acc);
-    sts(out + (size_t)(qa + t0 + tt) * C + c, silu_f(acc));
+    if (!(mode & 1)) acc = silu_f(acc);
+    if (mode & 2) acc += cur;
+    sts(out + (size_t)(qa + t0 + tt) * C + c, acc);
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS - 1; ++j) win[j] = j < taps - 2 ? win[j + 1] : j == taps - 2 ? cur : win[j];
   }
@@ -249,14 +253,14 @@ GRAG_API int grag_conv_max_taps() { return CONV_MAX_TAPS; }
 // update != 0: the pool is brought up to date after the convolution (one call per step and layer run)
 GRAG_API hipError_t grag_causal_conv(const void* proj, int ld, int coff, int C, int taps, const float* w, const float* b,
                                      void* cstate, const int* slots, const int* q_start, const int* ctx_len, void* out,
-                                     int nseq, int max_q_len, int nslots, int dt, hipStream_t st) {
+                                     int nseq, int max_q_len, int nslots, int dt, int mode, hipStream_t st) {
   if (nseq <= 0 || max_q_len <= 0) return hipSuccess;
   if (taps < 1 || taps > CONV_MAX_TAPS || C <= 0 || nseq > 65535) return hipErrorInvalidValue;
   const dim3 grid((C + 255) / 256, (max_q_len + CONV_TT - 1) / CONV_TT, nseq);
   if (grid.y > 65535) return hipErrorInvalidValue;
   DT_DISPATCH(dt, {
     hipLaunchKernelGGL(causal_conv_kernel<T>, grid, dim3(256), 0, st, (const T*)proj, ld, coff, C, taps, w, b,
-                       (const T*)cstate, slots, q_start, ctx_len, (T*)out, nslots);
+                       (const T*)cstate, slots, q_start, ctx_len, (T*)out, nslots, mode);
     if (taps > 1)
       hipLaunchKernelGGL(conv_state_kernel<T>, dim3((C + 255) / 256, nseq), dim3(256), 0, st, (const T*)proj, ld, coff, C,
                          taps, (T*)cstate, slots, q_start, ctx_len, nslots);

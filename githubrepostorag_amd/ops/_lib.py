@@ -79,11 +79,11 @@ _SIGS = {
     "grag_gemm_w4": [P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, P, P],
     "grag_gemm_w4_has": [I, I],
     "grag_err_alloc": [P],
-    "grag_embed_f32": [P, P, P, I, I, I, I, P],
+    "grag_embed_f32": [P, P, P, I, I, I, I, F, P],
     "grag_dyt_residual": [P, F, P, P, P, P, P, F, P, P, P, I, I, I, P],
     "grag_rope_vnorm_store": [P, I, I, I, I, P, P, I, P, P, P, P, I, I, I, I, I, I, I, ctypes.c_long, F, I, I, P],
-    "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P, P, I, I, P],
-    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, I, I, P, P, I, P, P, I, I, P],
+    "grag_sink_attn_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, F, I, I, I, P, P, I, I, I, F, P],
+    "grag_sink_attn_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, F, I, I, I, I, P, P, I, P, P, I, I, I, F, P],
     "grag_decay_attn_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, P, P, I, I, F, P],
     "grag_decay_attn_chunk": [],
     "grag_mingru_chunk": [],
@@ -94,21 +94,24 @@ _SIGS = {
     "grag_hyper_mix": [P, I, P, P, P, P, P, F, P, P, I, I, I, P],
     "grag_qk_norm_store": [P, I, I, I, P, P, P, P, P, P, I, I, I, I, I, ctypes.c_long, F, I, P],
     "grag_latent_store": [P, I, P, P, P, I, P, P, P, I, I, I, I, I, ctypes.c_long, F, I, P],
+    "grag_latent_rope_store": [P, I, I, I, P, P, P, I, P, P, P, I, I, I, I, I, ctypes.c_long, F, I, I, P],
+    "grag_tanh_cap": [P, I, I, I, F, I, P],
     "grag_sigmoid_window_prefill": [P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P, I, P],
     "grag_sigmoid_window_decode": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, I, I, P, I, P],
     "grag_rmsnorm_rows": [P, I, P, P, I, I, F, I, P],
     "grag_window_decode_mfma": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, I, P, I, P],
     "grag_attn_decode_xcd": [I],
     "grag_conv_max_taps": [],
-    "grag_causal_conv": [P, I, I, I, I, P, P, P, P, P, P, P, I, I, I, I, P],
+    "grag_causal_conv": [P, I, I, I, I, P, P, P, P, P, P, P, I, I, I, I, I, P],
     "grag_ssm_chunk": [],
     "grag_ssm_scan": [P, I, I, I, P, I, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, P, I, P],
     "grag_moe_max_rows": [],
     "grag_moe_max_top": [],
     "grag_moe_route": [P, I, P, I, I, I, I, I, I, P, P, P, I, I, P],
     "grag_moe_align": [P, I, I, P, P, P],
-    "grag_moe_gemm": [P, I, P, P, P, I, I, I, I, I, P, I, I, I, P],
-    "grag_residual_rmsnorm": [P, F, P, P, P, P, P, I, P, F, P, P, I, I, I, I, P],
+    "grag_moe_gemm": [P, I, P, P, P, I, I, I, I, I, P, I, I, I, F, F, F, P, I, P],
+    "grag_moe_table_route": [P, P, I, I, P, P, I, P],
+    "grag_residual_rmsnorm": [P, F, P, P, P, P, P, I, P, F, P, P, I, I, I, I, P, I, P, F, P],
 }
 
 

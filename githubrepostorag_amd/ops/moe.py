@@ -100,9 +100,6 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wgu: torch.Tensor, wd: torch
     return out
 
 
-_head_orders: dict = {}
-
-
 def head_project(x: torch.Tensor, w: torch.Tensor, gate: torch.Tensor | None = None) -> torch.Tensor:
     """One small matrix per head: x [T, H * K] (head h's K columns side by side), ``w`` [H, N, K] -> out [T, H * N] with
     out[t, h] = w[h] x[t, h]; with ``gate`` [T, H * N] (logits; rows may be a column slice of a wider tensor) the
@@ -116,19 +113,10 @@ def head_project(x: torch.Tensor, w: torch.Tensor, gate: torch.Tensor | None = N
             o = o * torch.sigmoid(gate.float())
         return o.to(x.dtype)
     assert x.is_contiguous() and x.shape[1] == H * K and w.is_contiguous() and w.dtype == x.dtype
-    assert gate is None or (gate.dtype == x.dtype and gate.stride(1) == 1 and gate.shape == (T, H * N)
-                            and gate.stride(0) % N == 0)
-    key = (T, H, str(x.device))
-    oo = _head_orders.get(key)
-    if oo is None:  # rows sorted by head: offs[h] = h T, order[h T + t] = t H + h
-        if len(_head_orders) > 64:
-            _head_orders.clear()
-        offs = (torch.arange(H + 1, dtype=torch.int32, device=x.device) * T).contiguous()
-        order = torch.arange(T * H, dtype=torch.int32, device=x.device).view(T, H).t().contiguous().view(-1)
-        oo = _head_orders[key] = (offs, order)
+    assert gate is None or (gate.dtype == x.dtype and gate.stride(1) == 1 and gate.shape == (T, H * N))
     out = torch.empty(T, H * N, dtype=x.dtype, device=x.device)
-    # rows of N (out) and K (x) numbers: row t H + h of x viewed [T H, K] is head h of token t; the gate's row
-    # t H + h starts gate_ld / N rows of N further per token
-    call("grag_moe_gemm", ptr(x), K, ptr(w), ptr(oo[0]), ptr(oo[1]), T * H, H, 1, N, K, ptr(out), N, 2, _dt(x),
+    # x viewed [T H, K] and out viewed [T H, N]: row t H + h is head h of token t.  The kernel's row order (sorted by
+    # head) follows from H and T alone, so it takes no offset / order arrays: `top` carries T
+    call("grag_moe_gemm", ptr(x), K, ptr(w), None, None, T * H, H, T, N, K, ptr(out), N, 2, _dt(x),
          float("inf"), 1.0, 0.0, ptr(gate), 0 if gate is None else gate.stride(0))
     return out
