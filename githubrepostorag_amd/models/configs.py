@@ -286,7 +286,7 @@ class HybridConfig:
                     if a.kv_from is None:
                         n += H * (a.kv_rank + a.rot_dim) + a.kv_rank
                 if L.mlp is not None:
-                    n += 1 + H * H + H + L.mlp.experts * 3 * H * L.mlp.ff
+                    n += 1 + H * H + H + L.mlp.experts * 3 * H * L.mlp.ff + self.vocab_size * L.mlp.top
             return n
         if self.arch == "leripel":
             n = 2 * self.vocab_size * H + H + (2 * H * H if self.loop_stop > self.loop_start else 0)

@@ -22,10 +22,6 @@ def scalar_norm(x, g, eps):
     return rms_unit(x, eps) * float(g)
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 def input_conv(h, w):
     """h + conv(h): per channel, tap j of w [width, taps] weighs the input taps - 1 - j steps back; nothing before
     the start of the sequence."""
@@ -73,12 +69,17 @@ def window_softmax(scores_of, i, window, sink=None):
     return lo, e / den
 
 
+def capped(z, cap):
+    """cap * tanh(z / cap); a cap of 0 (or none) leaves z as it is."""
+    return cap * torch.tanh(z / cap) if cap else z
+
+
 def attention(h, W, m):
     """Grouped-query sliding-window attention: rotary on halves of the first rot.dims of every q / k head, scores
     capped by softcap * tanh(score / softcap), plain softmax over the window.  h [T, width] -> [T, width]."""
     T = h.shape[0]
     H, G, d, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    win, scale, cap = m["mask"]["size"], m["scale"], m["softcap"]
+    win, scale, cap = m["mask"]["size"], m["scale"], m.get("softcap")
     rd, base = m["rot"]["dims"], m["rot"]["base"]
     q = (h @ W("q").T).view(T, H, d)
     k = (h @ W("k").T).view(T, G, d)
@@ -89,7 +90,7 @@ def attention(h, W, m):
         g = hh // (H // G)
         for i in range(T):
             qi = rotate_halves(q[i, hh], i, rd, base)
-            lo, p = window_softmax(lambda j: cap * torch.tanh((qi @ kr[j][g]) * scale / cap), i, win)
+            lo, p = window_softmax(lambda j: capped((qi @ kr[j][g]) * scale, cap), i, win)
             for n, j in enumerate(range(lo, i + 1)):
                 out[i, hh] += p[n] * v[j, g]
     return out.reshape(T, H * vd) @ W("o").T
@@ -161,7 +162,7 @@ def forward(cfg, sd, tokens, taps=None):
         p, m = f"l{i}.", L["mixer"]
         W = lambda n, p=p: P(p + "mix." + n)
         h = scalar_norm(x, P(p + "norm1"), eps)
-        hin = input_conv(h, P(p + "canon1"))
+        hin = input_conv(h, P(p + "canon1")) if cfg["canon"]["taps"] else h
         if L["type"] == "attention":
             y = attention(hin, W, m)
         else:
@@ -179,5 +180,82 @@ def forward(cfg, sd, tokens, taps=None):
         if taps is not None:
             taps.append(x.clone())
     z = scalar_norm(x, P("final.norm"), eps) @ P("head").T
-    cap = cfg["logit_softcap"]
-    return cap * torch.tanh(z / cap)
+    return capped(z, cfg.get("logit_softcap"))
+
+
+# ------------------------------------------------------------------------------------------------ test models
+def make_config(width=48, vocab=96, kinds=("attention", "latent", "attention", "shared"), no_mlp=(), heads=4,
+                kv_heads=2, dim=12, vdim=12, window=11, softcap=5.0, rot_dims=8, rot_base=100.0, scale=0.35,
+                lat_heads=3, lat_dim=8, lat_vdim=10, kv_rank=20, rot_dim=6, lat_window=19, lat_scale=0.3,
+                lat_base=50.0, experts=5, top=2, ff=24, limit=1.2, taps=3, eps=1e-5, embed_scale=2.5,
+                residual_mult=0.5, logit_softcap=12.0):
+    """A small config.json dict.  ``kinds``: "attention", "latent" (a latent layer with its own cache) or "shared" (a
+    latent layer that attends to the cache of the nearest "latent" before it)."""
+    layers, last = [], None
+    for i, kind in enumerate(kinds):
+        if kind == "attention":
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "softcap": softcap,
+                 "mask": {"size": window}, "rot": {"dims": rot_dims, "base": rot_base}}
+        else:
+            m = {"heads": lat_heads, "dim": lat_dim, "rot_dim": rot_dim, "vdim": lat_vdim, "kv_rank": kv_rank,
+                 "scale": lat_scale, "mask": {"size": lat_window}, "rot": {"dims": rot_dim, "base": lat_base}}
+            if kind == "shared":
+                m["kv_from"] = last
+            else:
+                last = i
+        mlp = None if i in no_mlp else {"kind": "moe", "expert": {"ff": ff, "limit": limit},
+                                        "router": {"experts": experts, "top": top}}
+        layers.append({"type": "attention" if kind == "attention" else "latent_attention", "mixer": m, "mlp": mlp})
+    return {"architecture": "Pubulix", "vocab": vocab, "width": width, "norm": {"eps": eps}, "canon": {"taps": taps},
+            "embedding": {"scale": embed_scale}, "residual_mult": residual_mult, "logit_softcap": logit_softcap,
+            "layers": layers}
+
+
+def make_weights(cfg, seed=0):
+    """Random bf16 weights (int32 tables) under the checkpoint's names."""
+    g = torch.Generator().manual_seed(4242 + seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def r(*shape, s=None):
+        s = shape[-1] ** -0.5 if s is None else s
+        return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16)
+
+    def num(v=1.0, s=0.15):
+        return (v + s * torch.randn((), generator=g)).to(torch.bfloat16)
+
+    sd = {"embed": r(V, W, s=1.0), "head": r(V, W, s=2.0 * W ** -0.5), "final.norm": num()}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        sd[p + "norm1"] = num()
+        if cfg["canon"]["taps"]:
+            sd[p + "canon1"] = r(W, cfg["canon"]["taps"], s=0.4)
+        sd[p + "rg1"], sd[p + "rg1.b"] = r(W, W), r(W, s=0.7)
+        if L["type"] == "attention":
+            H, G, d, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            sd.update({p + "mix.q": r(H * d, W, s=2.0 * W ** -0.5), p + "mix.k": r(G * d, W, s=2.0 * W ** -0.5),
+                       p + "mix.v": r(G * vd, W), p + "mix.o": r(W, H * vd)})
+        else:
+            H, d, rr, vd, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            sd.update({p + "mix.q": r(H * (d + rr), W, s=2.0 * W ** -0.5), p + "mix.uk": r(H * d, R),
+                       p + "mix.uv": r(H * vd, R), p + "mix.sink": r(H, s=1.5), p + "mix.g": r(H * vd, W),
+                       p + "mix.o": r(W, H * vd)})
+            if m.get("kv_from") is None:
+                sd[p + "mix.dkv"] = r(R + rr, W, s=2.0 * W ** -0.5)
+                sd[p + "mix.dkv.norm"] = (1.0 + 0.2 * torch.randn(R, generator=g)).to(torch.bfloat16)
+        f = L["mlp"]
+        if f is not None:
+            sd[p + "norm2"] = num()
+            sd[p + "rg2"], sd[p + "rg2.b"] = r(W, W), r(W, s=0.7)
+            E, F = f["router"]["experts"], f["expert"]["ff"]
+            for e in range(E):
+                sd.update({p + f"mlp.e{e}.gate": r(F, W, s=2.0 * W ** -0.5), p + f"mlp.e{e}.up": r(F, W, s=2.0 * W ** -0.5),
+                           p + f"mlp.e{e}.down": r(W, F)})
+            rows = [torch.randperm(E, generator=g)[: f["router"]["top"]] for _ in range(V)]
+            sd[p + "mlp.table"] = torch.stack(rows).to(torch.int32)
+    return sd
+
+
+def logits_and_taps(cfg, sd, tokens):
+    taps = []
+    z = forward(cfg, sd, tokens, taps)
+    return z, torch.stack(taps)
