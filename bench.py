@@ -174,9 +174,9 @@ def parse():
     ap.add_argument("--recall-queries", type=int, default=64,
                     help="queries per rank for recall@top-k of the IVF search vs an exact scan of every shard "
                          "(index_recall; 0: skip)")
-    ap.add_argument("--hybrid", nargs="?", const="zofesun", default=None, choices=("zofesun", "namudra", "leripel"),
+    ap.add_argument("--hybrid", nargs="?", const="zofesun", default=None, choices=("zofesun", "namudra", "leripel", "pubulix"),
                     help="instead of the headline workload: prefill / decode throughput of a hybrid decoder (zofesun, "
-                         "the default, namudra or leripel) beside the equal-size decoders the engine already serves, and a "
+                         "the default, namudra, leripel or pubulix) beside the equal-size decoders the engine already serves, and a "
                          "per-kernel roofline table (one GPU)")
     ap.add_argument("--out", default=None)
     args = ap.parse_args()

@@ -1,10 +1,12 @@
-"""``bench.py --hybrid [zofesun|namudra|leripel]``: prefill and decode throughput of a hybrid decoder beside the decoders of
+"""``bench.py --hybrid [zofesun|namudra|leripel|pubulix]``: prefill and decode throughput of a hybrid decoder beside the decoders of
 equal size that the engine already serves (same width, heads, head size, FFN width, layer count, vocabulary; random
 weights, synthetic token ids), all through LLMEngine.generate, and a per-kernel table: each new kernel and the
 like kernel of the closest model as a fraction of the roofline of what bounds it (HBM bytes or matrix / vector
 flops).  Zofesun stands beside Qwen2; Namudra beside Zofesun (the closest: fp32 residual, decay scan, sink
 attention kernels) and Qwen2; Leripel beside Namudra (the closest: fp32 residual, retention scan, the same attention
-kernel family, a layer list that is data) and Qwen2."""
+kernel family, a layer list that is data) and Qwen2; Pubulix beside Leripel (the closest: the same attention kernels
+with a window instead of blocks, experts on the same grouped GEMM, the same convolution and boundary kernels) and
+Qwen2, with Namudra's latent attention as the like kernel of its latent layers."""
 from __future__ import annotations
 
 import json
@@ -430,6 +432,184 @@ def _leripel_kernel_table(dev, H=28, G=4, D=128, W=3584, ff=18944, T=2048, B=64,
     return rows
 
 
+def _pubulix_models(name, dev):
+    """Pubulix at a bench size: per four layers capped sliding-window attention (window 1024), latent attention with
+    its own cache (window 2048), attention again, latent attention over the same cache; every layer with 16
+    table-routed experts (4 per token) whose active width equals the dense decoders' feed-forward, an input
+    convolution of 4 taps and gated residual branches; beside the Leripel and Qwen2 stacks."""
+    from ..models.configs import pubulix_config
+    from ..models.pubulix import PubulixModel
+
+    W, H, G, D, ff, nl, _ = SIZES[name]
+    pc = pubulix_config(f"pubulix-{name}", VOCAB, W, ("alas" * nl)[:nl], heads=H, kv_heads=G, dim=D, window=1024,
+                        lat_heads=H, kv_rank=192, rot_dim=64, lat_window=2048, experts=16, top=4, ff=(ff // 4) // 64 * 64)
+    mk_l, _, mk_q = _leripel_models(name, dev)
+    return (lambda: PubulixModel(pc, device=dev, seed=1)), mk_l, mk_q
+
+
+def _pubulix_kernel_table(dev, H=28, G=4, D=128, W=3584, ff=18944, T=2048, B=64, ctx=2048, bs=16, win=1024, lwin=2048,
+                          R=192, r=64, E=16, top=4, V=VOCAB):
+    """[(kernel, seconds, bound, fraction of roofline)] for Pubulix's kernels and the like kernels of Leripel (attention,
+    convolution, boundary, experts) and Namudra (latent attention)."""
+    from ..ops.attention import AttnMetadata, sink_attention
+    from ..ops.elementwise import latent_rope_store, latent_store, rope_table, tanh_cap_
+    from ..ops.linear import linear
+    from ..ops.moe import head_project, moe_experts, moe_route, moe_table_route
+    from ..ops.norm import residual_rmsnorm
+    from ..ops.recurrent import causal_conv
+
+    bf = torch.bfloat16
+    i32 = dict(dtype=torch.int32, device=dev)
+    rows = []
+
+    def add(name, sec, flops=0.0, bytes_=0.0, peak=MFMA_BF16):
+        t_c, t_m = flops / peak, bytes_ / HBM_BPS
+        rows.append({"kernel": name, "us": round(sec * 1e6, 1), "bound": "flops" if t_c >= t_m else "bytes",
+                     "roofline_fraction": round(max(t_c, t_m) / sec, 4)})
+
+    nb = T // bs
+    meta = AttnMetadata(q_start=torch.tensor([0, T], **i32), ctx_len=torch.tensor([T], **i32),
+                        block_tables=(torch.arange(nb, **i32) + 1).view(1, nb), slot_mapping=torch.arange(T, **i32) + bs,
+                        max_q_len=T, num_seqs=1, num_tokens=T, state_slots=torch.tensor([0], **i32))
+    nbd = ctx // bs
+    dmeta = AttnMetadata(q_start=torch.arange(B + 1, **i32), ctx_len=torch.full((B,), ctx, **i32),
+                         block_tables=(torch.arange(B * nbd, **i32) + 1).view(B, nbd), slot_mapping=None, max_q_len=1,
+                         num_seqs=B, num_tokens=B, is_decode=True, state_slots=torch.arange(B, **i32))
+    # ---- attention: a window of `win` positions with capped scores | leripel's blocks of the same length
+    kc = torch.randn(nb + 1, G, bs, D, device=dev).to(bf)
+    vc = torch.randn(nb + 1, G, bs, D, device=dev).to(bf)
+    q = torch.randn(T, H, D, device=dev).to(bf)
+    temp = torch.ones(H, device=dev)
+    hg = torch.randn(T, H, device=dev).to(bf)
+    pairs_w = T * (T + 1) / 2 - (T - win) * (T - win + 1) / 2
+    pairs_c = (T // win) * win * (win + 1) / 2
+    add(f"capped window attention prefill (window {win})",
+        _timed(lambda: sink_attention(q, kc, vc, meta, 0.09, None, window=win, softcap=50.0)), flops=4.0 * pairs_w * H * D)
+    add(f"leripel block-local attention prefill (blocks of {win})",
+        _timed(lambda: sink_attention(q, kc, vc, meta, 0.09, None, head_scale=temp, head_gate=hg, chunk=win)),
+        flops=4.0 * pairs_c * H * D)
+    kd = torch.randn(B * nbd + 1, G, bs, D, device=dev).to(bf)
+    vd_ = torch.randn(B * nbd + 1, G, bs, D, device=dev).to(bf)
+    qd = torch.randn(B, H, D, device=dev).to(bf)
+    hgd = torch.randn(B, H, device=dev).to(bf)
+    add(f"capped window attention decode ({win} keys)",
+        _timed(lambda: sink_attention(qd, kd, vd_, dmeta, 0.09, None, window=win, softcap=50.0)),
+        bytes_=2.0 * B * win * G * D * 2)
+    add(f"leripel block-local attention decode ({win} keys)",
+        _timed(lambda: sink_attention(qd, kd, vd_, dmeta, 0.09, None, head_scale=temp, head_gate=hgd, chunk=win)),
+        bytes_=2.0 * B * win * G * D * 2)
+    # ---- latent attention: a window and a sink over latent | rotated rows | namudra's causal form on the same rows
+    lk = torch.randn(nb + 1, 1, bs, R + r, device=dev).to(bf)
+    lq = torch.randn(T, H, R + r, device=dev).to(bf)
+    sink = torch.zeros(H, device=dev)
+    pairs_l = T * (T + 1) / 2 - max(0, T - lwin) * (max(0, T - lwin) + 1) / 2
+    add(f"latent attention prefill (window {lwin}, sink)",
+        _timed(lambda: sink_attention(lq, lk, lk[..., :R], meta, 0.06, sink, window=lwin)),
+        flops=2.0 * pairs_l * H * (2 * R + r))
+    add("namudra latent attention prefill (causal)", _timed(lambda: sink_attention(lq, lk, lk[..., :R], meta, 0.06, None)),
+        flops=2.0 * (T * (T + 1) / 2) * H * (2 * R + r))
+    lkd = torch.randn(B * nbd + 1, 1, bs, R + r, device=dev).to(bf)
+    lqd = torch.randn(B, H, R + r, device=dev).to(bf)
+    add(f"latent attention decode ({min(ctx, lwin)} keys, sink)",
+        _timed(lambda: sink_attention(lqd, lkd, lkd[..., :R], dmeta, 0.06, sink, window=lwin)),
+        bytes_=1.0 * B * min(ctx, lwin) * (R + r) * 2)
+    add(f"namudra latent attention decode ({ctx} keys)",
+        _timed(lambda: sink_attention(lqd, lkd, lkd[..., :R], dmeta, 0.06, None)), bytes_=1.0 * B * ctx * (R + r) * 2)
+    # ---- queries + cache row out of the fused projection | namudra's in-place form
+    ld = H * (R + r) + (R + r) + H * D
+    proj = torch.randn(T, ld, device=dev).to(bf)
+    pos = torch.arange(T, **i32)
+    tab = rope_table(T, r, 1e4, dev)
+    cw = torch.ones(R, device=dev)
+    add("latent_rope_store (queries copied and rotated, cache row)", _timed(lambda: latent_rope_store(
+        proj, 0, H * (R + r), cw, pos, tab, meta.slot_mapping, lk, H, 1e-5, interleaved=True)),
+        bytes_=T * (H + 1) * (R + r) * 2 * 2.0)
+    ckv = torch.randn(T, R + r, device=dev).to(bf)
+    add("namudra latent_store (queries rotated in place)", _timed(lambda: latent_store(ckv, cw, pos, tab, meta.slot_mapping,
+                                                                                        lq, lk, 1e-5)),
+        bytes_=T * (R + r) * 2 * 2.0 + T * H * r * 2 * 2.0)
+    # ---- one value matrix per head + gate | one dense GEMM of the same flops through linear()
+    o = torch.randn(T, H * R, device=dev).to(bf)
+    wuv = (torch.randn(H, D, R, device=dev) * 0.05).to(bf)
+    gcol = proj[:, H * (R + r) + (R + r):]
+    add(f"head_project prefill ({H} matrices {D} x {R}, gate)", _timed(lambda: head_project(o, wuv, gate=gcol)),
+        flops=2.0 * T * H * D * R, bytes_=T * H * (R + 2 * D) * 2.0)
+    wdn = (torch.randn(D, H * R, device=dev) * 0.02).to(bf)
+    add("dense GEMM of the same flops (linear)", _timed(lambda: linear(o, wdn)), flops=2.0 * T * H * D * R,
+        bytes_=T * H * R * 2.0)
+    od = torch.randn(B, H * R, device=dev).to(bf)
+    gd = torch.randn(B, H * D, device=dev).to(bf)
+    add("head_project decode rows", _timed(lambda: head_project(od, wuv, gate=gd)), bytes_=H * D * R * 2.0)
+    add("dense GEMM of the same weight bytes, decode rows (linear)", _timed(lambda: linear(od, wdn)), bytes_=H * D * R * 2.0)
+    # ---- sublayer boundary: gated branch | leripel's ungated sum of the same operands
+    x = torch.randn(T, W, device=dev)
+    a = torch.randn(T, W, device=dev).to(bf)
+    gt = torch.randn(T, W, device=dev).to(bf)
+    e = torch.randn(T, top, W, device=dev).to(bf)
+    ec, gb, w32 = torch.rand(T, top, device=dev), torch.zeros(W, device=dev), torch.ones(W, device=dev)
+    add("residual_rmsnorm (gated mixer branch)", _timed(lambda: residual_rmsnorm(x, a, w=w32, eps=1e-5, gate=gt, gbias=gb, mult=0.5)),
+        bytes_=T * W * (8 + 2.0 * 2 + 2))
+    add("leripel residual_rmsnorm (one branch)", _timed(lambda: residual_rmsnorm(x, a, w=w32, eps=1e-5)),
+        bytes_=T * W * (8 + 2.0 + 2))
+    add(f"residual_rmsnorm (gated sum of {top} experts)",
+        _timed(lambda: residual_rmsnorm(x, e=e, ecoef=ec, w=w32, eps=1e-5, gate=gt, gbias=gb, mult=0.5)),
+        bytes_=T * W * (8 + 2.0 * (1 + top) + 2))
+    add(f"leripel residual_rmsnorm (sum of {top} experts)", _timed(lambda: residual_rmsnorm(x, e=e, ecoef=ec, w=w32, eps=1e-5)),
+        bytes_=T * W * (8 + 2.0 * top + 2))
+    # ---- input convolution (no activation, input added) | leripel's SiLU form over the same channels
+    h = torch.randn(T, W, device=dev).to(bf)
+    cwt = torch.randn(W, 4, device=dev) * 0.3
+    cst = torch.zeros(B + 1, 3, W, device=dev, dtype=bf)
+    add("input convolution prefill (4 taps, h + conv(h))", _timed(lambda: causal_conv(h, 0, cwt, None, cst, meta, act=False, residual=True)),
+        bytes_=T * W * 2 * 2.0)
+    add("leripel causal_conv prefill (4 taps, SiLU)", _timed(lambda: causal_conv(h, 0, cwt, None, cst, meta)), bytes_=T * W * 2 * 2.0)
+    hd = torch.randn(B, W, device=dev).to(bf)
+    add("input convolution decode", _timed(lambda: causal_conv(hd, 0, cwt, None, cst, dmeta, act=False, residual=True)),
+        bytes_=B * W * 2 * (2 + 2 * 3.0))
+    add("leripel causal_conv decode", _timed(lambda: causal_conv(hd, 0, cwt, None, cst, dmeta)), bytes_=B * W * 2 * (2 + 2 * 3.0))
+    # ---- experts: table routing, clamped units | leripel's router and SiLU units on the same grouped GEMM
+    F = (ff // 4) // 64 * 64
+    table = torch.rand(V, E, device=dev).argsort(1)[:, :top].to(torch.int32).contiguous()
+    tok = torch.randint(0, V, (T,), device=dev).to(torch.int32)
+    wr = torch.randn(E, W, device=dev) * 0.05
+    add("moe_table_route", _timed(lambda: moe_table_route(tok, table)), bytes_=T * (4 + top * 12.0))
+    add("leripel moe_route (16 experts)", _timed(lambda: moe_route(h, wr, E, top, 4, 2)), flops=2.0 * T * E * W, bytes_=T * W * 2.0,
+        peak=VALU_F32)
+    ids, _ = moe_table_route(tok, table)
+    wgu = (torch.randn(E, 2 * F, W, device=dev) * 0.02).to(bf)
+    wd = (torch.randn(E, W, F, device=dev) * 0.02).to(bf)
+    add(f"clamped experts prefill ({T} x {top} rows)", _timed(lambda: moe_experts(h, ids, wgu, wd, 7.0, 1.702, 1.0)),
+        flops=6.0 * T * top * F * W)
+    add(f"leripel SiLU experts prefill ({T} x {top} rows)", _timed(lambda: moe_experts(h, ids, wgu, wd)), flops=6.0 * T * top * F * W)
+    idd, _ = moe_table_route(tok[:B].contiguous(), table)
+    add(f"clamped experts decode ({B} x {top} rows)", _timed(lambda: moe_experts(hd, idd, wgu, wd, 7.0, 1.702, 1.0)),
+        bytes_=3.0 * E * F * W * 2)
+    add(f"leripel SiLU experts decode ({B} x {top} rows)", _timed(lambda: moe_experts(hd, idd, wgu, wd)), bytes_=3.0 * E * F * W * 2)
+    # ---- logit cap
+    lg = torch.randn(B, V, device=dev).to(bf)
+    add(f"tanh_cap ({B} x {V} logits)", _timed(lambda: tanh_cap_(lg, 30.0)), bytes_=B * V * 2 * 2.0)
+    return rows
+
+
+def run_pubulix(args) -> dict:
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    sizes = {}
+    for name in SIZES:
+        makers = dict(zip(("pubulix", "leripel", "qwen2"), _pubulix_models(name, dev)))
+        cell = {}
+        for batch, plen, glen in ((8, 2048, 64), (64, 1024, 64)):
+            key = f"B{batch}_P{plen}_G{glen}"
+            cell[key] = {k: _engine_numbers(mk, dev, batch, plen, glen) for k, mk in makers.items()}
+            print(json.dumps({"size": name, "shape": key, **cell[key]}), flush=True)
+        sizes[name] = cell
+    kernels = _pubulix_kernel_table(dev)
+    for r in kernels:
+        print(json.dumps(r), flush=True)
+    return {"metric": "pubulix_vs_leripel_vs_qwen2_tokens_per_s", "unit": "tokens/s", "dtype": "bf16",
+            "data": "synthetic", "sizes": sizes, "kernels": kernels}
+
+
 def run_leripel(args) -> dict:
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
@@ -473,6 +653,8 @@ def run(args) -> dict:
         return run_namudra(args)
     if getattr(args, "hybrid", None) == "leripel":
         return run_leripel(args)
+    if getattr(args, "hybrid", None) == "pubulix":
+        return run_pubulix(args)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     sizes = {}
