@@ -23,7 +23,7 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); 
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
 // ------------------------------------------------------------------------------------------------ causal convolution
-constexpr int CONV_MAX_TAPS = 8;
+constexpr int CONV_MAX_TAPS = 16;
 constexpr int CONV_TT = 16;  // tokens per workgroup
 
 // out [T][C] = SiLU(b[c] + sum_j w[c][j] in[t - (taps - 1) + j][c]), in = proj columns coff .. coff + C; inputs before
