@@ -198,6 +198,11 @@ def case_other_sizes(device, tol, dtype=torch.float32):
         # a wide latent (more than 64 value columns per lane chunk) and a long head
         dict(width=64, kinds=("latent", "shared"), lat_heads=2, lat_dim=16, lat_vdim=8, kv_rank=136, rot_dim=8,
              lat_window=23, no_mlp=(0, 1)),
+        # a width and a vocabulary that are multiples of nothing useful (rows of 60 and 72 bytes), odd head sizes
+        dict(width=30, vocab=77, kinds=("attention", "latent", "shared"), heads=2, kv_heads=1, dim=10, vdim=6,
+             rot_dims=6, lat_heads=2, lat_dim=5, lat_vdim=7, kv_rank=11, rot_dim=2, ff=9, experts=2, top=2, taps=4),
+        dict(width=36, vocab=101, kinds=("latent", "attention"), heads=6, kv_heads=3, dim=6, vdim=10, rot_dims=2,
+             lat_heads=4, lat_dim=6, lat_vdim=6, kv_rank=18, rot_dim=6, ff=20, experts=7, top=4, taps=2),
     ]
     for i, kw in enumerate(variants):
         cfg = O.make_config(**kw)
