@@ -252,15 +252,17 @@ moe_align_kernel(const int* __restrict__ ids, int n, int E, int* __restrict__ of
 }
 
 // ------------------------------------------------------------------------------------------------ table routing
-// ids [T][top] <- table [vocab][top] row of every token id, wts [T][top] <- 1 / top.  One thread per (token, choice).
+// ids [nl][T][top] <- table [nl][vocab][top] row of every token id (nl layers' tables in one launch), wts [T][top] <-
+// 1 / top.  One thread per (token, choice); grid.y = layer.
 __global__ void moe_table_route_kernel(const int* __restrict__ tok, const int* __restrict__ table, int vocab, int top,
                                        int* __restrict__ ids, float* __restrict__ wts, int n) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   const int t = i / top, k = i - t * top;
   const int id = tok[t];
-  ids[i] = index_ok(id, vocab, ERR_EMBED_TOKEN) ? table[(size_t)id * top + k] : -1;  // (-1: the pair is skipped)
-  wts[i] = 1.f / (float)top;
+  const int* tab = table + (size_t)blockIdx.y * vocab * top;
+  ids[(size_t)blockIdx.y * n + i] = index_ok(id, vocab, ERR_EMBED_TOKEN) ? tab[(size_t)id * top + k] : -1;  // (-1: the pair is skipped)
+  if (blockIdx.y == 0) wts[i] = 1.f / (float)top;
 }
 
 // ------------------------------------------------------------------------------------------------ grouped GEMM
@@ -767,12 +769,12 @@ GRAG_API hipError_t grag_moe_align(const int* ids, int n, int E, int* offs, int*
   return hipGetLastError();
 }
 
-GRAG_API hipError_t grag_moe_table_route(const int* tok, const int* table, int vocab, int top, int* ids, float* wts,
-                                         int T_, hipStream_t st) {
-  if (T_ <= 0) return hipSuccess;
-  if (top < 1 || vocab < 1) return hipErrorInvalidValue;
+GRAG_API hipError_t grag_moe_table_route(const int* tok, const int* table, int nl, int vocab, int top, int* ids,
+                                         float* wts, int T_, hipStream_t st) {
+  if (T_ <= 0 || nl <= 0) return hipSuccess;
+  if (top < 1 || vocab < 1 || nl > 65535) return hipErrorInvalidValue;
   const int n = T_ * top;
-  hipLaunchKernelGGL(moe_table_route_kernel, dim3((n + 255) / 256), dim3(256), 0, st, tok, table, vocab, top, ids, wts, n);
+  hipLaunchKernelGGL(moe_table_route_kernel, dim3((n + 255) / 256, nl), dim3(256), 0, st, tok, table, vocab, top, ids, wts, n);
   return hipGetLastError();
 }
 

@@ -28,12 +28,14 @@ constexpr int CONV_TT = 16;  // tokens per workgroup
 
 // out [T][C] = SiLU(b[c] + sum_j w[c][j] in[t - (taps - 1) + j][c]), in = proj columns coff .. coff + C; inputs before
 // the portion come from cstate [slots][taps - 1][C] (oldest first), zeros for a sequence that starts at position 0.
-// mode bit 0: no SiLU; bit 1: the token's own input is added to the result (in + conv(in)).
-// grid (ceil(C / 256), ceil(max_q_len / CONV_TT), nseq).  The pool is only read here.
+// mode bit 0: no SiLU; bit 1: the token's own input is added to the result (in + conv(in)); bit 2 (only when one token
+// tile holds every portion, gridDim.y == 1): the thread, which then walks ALL tokens of its (sequence, channel), also
+// leaves the last taps - 1 inputs in the pool -- they are the window it ends with -- and no second kernel runs.
+// grid (ceil(C / 256), ceil(max_q_len / CONV_TT), nseq).  Without bit 2 the pool is only read here.
 template <typename T>
 __global__ void __launch_bounds__(256)
 causal_conv_kernel(const T* __restrict__ proj, int ld, int coff, int C, int taps, const float* __restrict__ w,
-                   const float* __restrict__ b, const T* __restrict__ cstate, const int* __restrict__ slots,
+                   const float* __restrict__ b, T* __restrict__ cstate, const int* __restrict__ slots,
                    const int* __restrict__ q_start, const int* __restrict__ ctx_len, T* __restrict__ out, int nslots,
                    int mode) {
   const int seq = blockIdx.z, c = blockIdx.x * 256 + threadIdx.x;
@@ -72,6 +74,12 @@ causal_conv_kernel(const T* __restrict__ proj, int ld, int coff, int C, int taps
     sts(out + (size_t)(qa + t0 + tt) * C + c, acc);
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS - 1; ++j) win[j] = j < taps - 2 ? win[j + 1] : j == taps - 2 ? cur : win[j];
+  }
+  if ((mode & 4) && taps > 1 && index_ok(slot, nslots, ERR_SAMPLER_SLOT)) {
+    T* dst = cstate + (size_t)slot * (taps - 1) * C;
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS - 1; ++j)
+      if (j < taps - 1) sts(dst + (size_t)j * C + c, win[j]);
   }
 }
 
@@ -258,10 +266,12 @@ GRAG_API hipError_t grag_causal_conv(const void* proj, int ld, int coff, int C, 
   if (taps < 1 || taps > CONV_MAX_TAPS || C <= 0 || nseq > 65535) return hipErrorInvalidValue;
   const dim3 grid((C + 255) / 256, (max_q_len + CONV_TT - 1) / CONV_TT, nseq);
   if (grid.y > 65535) return hipErrorInvalidValue;
+  const bool one_tile = grid.y == 1;  // every portion in one token tile: the convolution's threads update the pool
+  mode = (mode & 3) | (one_tile ? 4 : 0);
   DT_DISPATCH(dt, {
     hipLaunchKernelGGL(causal_conv_kernel<T>, grid, dim3(256), 0, st, (const T*)proj, ld, coff, C, taps, w, b,
-                       (const T*)cstate, slots, q_start, ctx_len, (T*)out, nslots, mode);
-    if (taps > 1)
+                       (T*)cstate, slots, q_start, ctx_len, (T*)out, nslots, mode);
+    if (taps > 1 && !one_tile)
       hipLaunchKernelGGL(conv_state_kernel<T>, dim3((C + 255) / 256, nseq), dim3(256), 0, st, (const T*)proj, ld, coff, C,
                          taps, (T*)cstate, slots, q_start, ctx_len, nslots);
   })

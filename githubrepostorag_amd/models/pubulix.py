@@ -152,7 +152,9 @@ class PubulixModel:
             return expect(name, *shape).to(device=dev, dtype=torch.float32).contiguous()
 
         def scalar_norm(name):  # one number for all coordinates: spread to the row the norm kernels multiply by
-            return torch.full((W,), float(expect(name).float()), dtype=torch.float32, device=dev)
+            if name not in sd or sd[name].numel() != 1:
+                raise ValueError(f"{name}: expected one number")
+            return torch.full((W,), float(sd[name].float().reshape(())), dtype=torch.float32, device=dev)
 
         self.embed = act(expect("embed", cfg.vocab_size, W))
         # LM head rows padded to a multiple of 8: the sampler reads logit rows 8 at a time (zero rows, cut off
@@ -210,6 +212,17 @@ class PubulixModel:
                                          for e in range(f.experts)], 0))
                 L.wd = act(torch.stack([expect(f_ + f"e{e}.down", W, f.ff) for e in range(f.experts)], 0))
             self.layers.append(L)
+        # the tables of all layers with the same number of choices side by side: one routing launch per step serves
+        # them all (a layer's tables entry becomes (stack, row))
+        groups: dict = {}
+        for L in self.layers:
+            if L.table is not None:
+                groups.setdefault(L.table.shape[1], []).append(L)
+        self.route_tables = {}
+        for top, Ls in groups.items():
+            self.route_tables[top] = torch.stack([L.table for L in Ls], 0).contiguous()
+            for k, L in enumerate(Ls):
+                L.table = (top, k)
 
     def prepare(self, max_len: int) -> None:
         """Rotary tables for positions below ``max_len`` (the engine calls this with its max_model_len before any
@@ -225,7 +238,7 @@ class PubulixModel:
     def param_bytes(self) -> int:
         n = 0
         for t in [self.embed, self.head] + [x for L in self.layers
-                                            for x in (L.wp, L.wo, L.wuv, L.rg1, L.rg2, L.wgu, L.wd, L.table)]:
+                                            for x in (L.wp, L.wo, L.wuv, L.rg1, L.rg2, L.wgu, L.wd)] + list(self.route_tables.values()):
             if t is not None:
                 n += t.numel() * t.element_size()
         return n
@@ -302,6 +315,7 @@ class PubulixModel:
         dt, eps, mult = self.dtype, cfg.norm_eps, cfg.residual_mult
         ids = input_ids.to(torch.int32).contiguous()
         x = embed_gather_f32(ids, self.embed, cfg.embed_scale)
+        routes = {top: moe_table_route(ids, t) for top, t in self.route_tables.items()}  # every layer's experts
         pend = {}  # the previous sublayer's output and gate, added at the next boundary
         for ri, (li, _, _) in enumerate(self.runs):
             L = self.layers[li]
@@ -312,7 +326,7 @@ class PubulixModel:
             f = L.spec.mlp
             if f is not None:
                 h = residual_rmsnorm(x, **pend, w=L.norm2, eps=eps, out_dtype=dt)
-                eids, wts = moe_table_route(ids, L.table)
+                eids, wts = routes[L.table[0]][0][L.table[1]], routes[L.table[0]][1]
                 e = moe_experts(h, eids, L.wgu, L.wd, f.limit, EXPERT_ALPHA, EXPERT_SHIFT)
                 pend = {"e": e, "ecoef": wts, "gate": linear(h, L.rg2), "gbias": L.rg2b, "mult": mult}
             if taps is not None:

@@ -110,7 +110,7 @@ _SIGS = {
     "grag_moe_route": [P, I, P, I, I, I, I, I, I, P, P, P, I, I, P],
     "grag_moe_align": [P, I, I, P, P, P],
     "grag_moe_gemm": [P, I, P, P, P, I, I, I, I, I, P, I, I, I, F, F, F, P, I, P],
-    "grag_moe_table_route": [P, P, I, I, P, P, I, P],
+    "grag_moe_table_route": [P, P, I, I, I, P, P, I, P],
     "grag_residual_rmsnorm": [P, F, P, P, P, P, P, I, P, F, P, P, I, I, I, I, P, I, P, F, P],
 }
 

@@ -452,6 +452,10 @@ def sink_attention_ref(q, k_cache, v_cache, meta: AttnMetadata, scale: float, si
     return out
 
 
+# windowed decode: with at most this many (sequence, kv head) workgroups the step's key splits are taken also for
+# windows of <= 1024 keys (the parts wholly before the window exit at once; 8 sequences x 4 kv heads, window 1024:
+# 47 -> 26 us with 256-key parts), above it one workgroup walks the window (64 x 4: 56 us against 70 with parts)
+WINDOW_SPLIT_ROWS = int(os.environ.get("GRAG_WINDOW_SPLIT_ROWS", "64"))
 NO_SINK = -1.0e30  # a sink logit this low adds exactly 0 to the denominator once any key is seen: plain softmax
 _no_sinks: dict = {}
 
@@ -517,8 +521,11 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     if meta.is_decode and meta.max_q_len == 1:
         # key splits (flash-decoding) when the step brings a plan and scratch that holds it
         nsplit = meta.num_splits
-        if 0 < chunk <= 1024 or 0 < window <= 1024:  # the visible keys are few: one workgroup per (sequence, kv head)
+        if 0 < chunk <= 1024:  # a block's keys are few: one workgroup per (sequence, kv head) walks them
             nsplit = 1
+        if 0 < window <= 1024 and (meta.num_seqs * G * ((H // G + 15) // 16) > WINDOW_SPLIT_ROWS
+                                   or window <= 2 * meta.split_len):
+            nsplit = 1  # enough (sequence, kv head) rows for the chip, or a window of a part or two: one pass, no combine
         if (nsplit > 1 and (meta.part_o is None or meta.part_ml is None
                             or meta.part_o.numel() < nsplit * meta.num_seqs * H * vd
                             or meta.part_ml.numel() < nsplit * meta.num_seqs * H * 2)):

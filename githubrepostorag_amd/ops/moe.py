@@ -49,15 +49,17 @@ def moe_route(h: torch.Tensor, wr: torch.Tensor, E: int, top: int, groups: int =
 
 def moe_table_route(token_ids: torch.Tensor, table: torch.Tensor):
     """Routing without a router: ``table`` [vocab, top] int32 names the experts of every token id.  Returns
-    (ids [T, top] int32 = the rows of the step's token ids, wts [T, top] fp32 = 1 / top each)."""
-    T, top = token_ids.numel(), table.shape[1]
+    (ids [T, top] int32 = the rows of the step's token ids, wts [T, top] fp32 = 1 / top each).  ``table``
+    [layers, vocab, top]: the tables of several layers in one launch, ids [layers, T, top]."""
+    T, top = token_ids.numel(), table.shape[-1]
     if not table.is_cuda:
-        ids = table[token_ids.long()].to(torch.int32).contiguous()
+        ids = table[..., token_ids.long(), :].to(torch.int32).contiguous()
         return ids, torch.full((T, top), 1.0 / top, dtype=torch.float32)
     assert table.dtype == torch.int32 and table.is_contiguous() and token_ids.dtype == torch.int32
-    ids = torch.empty(T, top, dtype=torch.int32, device=table.device)
+    nl = 1 if table.dim() == 2 else table.shape[0]
+    ids = torch.empty(*table.shape[:-2], T, top, dtype=torch.int32, device=table.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=table.device)
-    call("grag_moe_table_route", ptr(token_ids), ptr(table), table.shape[0], top, ptr(ids), ptr(wts), T)
+    call("grag_moe_table_route", ptr(token_ids), ptr(table), nl, table.shape[-2], top, ptr(ids), ptr(wts), T)
     return ids, wts
 
 

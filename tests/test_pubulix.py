@@ -140,6 +140,10 @@ def table_experts_case(device, dtype, tol):
         tok = torch.randint(0, V, (T,), generator=g).to(torch.int32)
         ids, wts = moe_table_route(tok.to(device), table.to(device))
         assert torch.equal(ids.cpu(), table[tok.long()]) and float((wts.cpu() - 1.0 / top).abs().max()) < 1e-7
+        both = torch.stack([table, table.flip(0)]).contiguous()  # two layers' tables in one call
+        ids2, wts2 = moe_table_route(tok.to(device), both.to(device))
+        assert torch.equal(ids2[0].cpu(), table[tok.long()]) and torch.equal(ids2[1].cpu(), table.flip(0)[tok.long()])
+        assert torch.equal(wts2.cpu(), wts.cpu())
         e = moe_experts(h.to(device), ids, wgu.to(device), wd.to(device), limit, 1.702, 1.0)
         x = torch.zeros(T, W, device=device)
         residual_rmsnorm(x, e=e, ecoef=wts, out_dtype=dtype)

@@ -148,6 +148,19 @@ def test_serving_head_sizes():
     assert C.rel_err(C.feed_in_portions(eng, "d", toks, [70, 64] + [1] * 16), want) < F32
 
 
+def test_many_heads_on_one_latent():
+    """More than 16 heads share the one cached row of a latent layer: the decode kernel packs them 16 to a
+    workgroup; with a window, sinks and key splits, both precisions."""
+    cfg = O.make_config(width=64, kinds=("latent", "shared"), no_mlp=(0, 1), lat_heads=20, lat_dim=16, lat_vdim=16,
+                        kv_rank=32, rot_dim=16, lat_window=90)
+    sd = O.make_weights(cfg, seed=61)
+    toks = C.tokens(cfg, 160, 13)
+    want = O.forward(cfg, sd, toks)
+    for dtype, tol in ((torch.bfloat16, BF16), (torch.float32, F32)):
+        _, eng = C.build(cfg, sd, "cuda", dtype)
+        assert C.rel_err(C.feed_in_portions(eng, "m", toks, [100, 33] + [1] * 27), want) < tol
+
+
 def test_key_splits_with_windows():
     """Windows longer than the decode kernel's single-pass limit take the engine's key splits: splits that lie wholly
     before the query's window are empty, the split that holds the window's oldest key starts inside it."""
@@ -159,6 +172,15 @@ def test_key_splits_with_windows():
     want = O.forward(cfg, sd, toks)
     _, eng = C.build(cfg, sd, "cuda", torch.bfloat16, pool_tokens=1408)
     assert C.rel_err(C.feed_in_portions(eng, "k", toks, [1090] + [1] * 20 + [170] + [1] * 20), want) < BF16
+    # windows below the single-pass limit take the splits too when few sequences decode: parts before the window are
+    # empty, the window starts inside a part
+    cfg = O.make_config(width=64, kinds=("attention", "latent"), no_mlp=(0, 1), heads=4, kv_heads=2, dim=16, vdim=16,
+                        scale=0.4, window=700, rot_dims=8, lat_heads=2, lat_dim=16, lat_vdim=16, kv_rank=32, rot_dim=16,
+                        lat_window=900)
+    sd = O.make_weights(cfg, seed=60)
+    want = O.forward(cfg, sd, toks)
+    _, eng = C.build(cfg, sd, "cuda", torch.bfloat16, pool_tokens=1408)
+    assert C.rel_err(C.feed_in_portions(eng, "s", toks, [1250] + [1] * 50), want) < BF16
 
 
 @pytest.mark.parametrize("graphs,mixed,window,max_batched", [(False, False, 1, 4096), (True, False, 1, 4096),
