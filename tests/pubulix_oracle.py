@@ -58,15 +58,12 @@ def rotate_halves(vec, pos, dims, base):
     return out
 
 
-def window_softmax(scores_of, i, window, sink=None):
-    """Weights of the keys j = max(0, i - window + 1) .. i for query i; ``sink``: one more term exp(sink) in the
-    denominator that belongs to no key.  -> (first key, weights)."""
-    lo = max(0, i - window + 1)
-    sc = torch.stack([scores_of(j) for j in range(lo, i + 1)])
-    m = sc.max() if sink is None else torch.maximum(sc.max(), torch.as_tensor(float(sink), dtype=F64))
-    e = torch.exp(sc - m)
-    den = e.sum() + (0.0 if sink is None else math.exp(float(sink) - float(m)))
-    return lo, e / den
+def window_softmax(scores, sink=None):
+    """Softmax over the scores of a query's visible keys; ``sink``: one more term exp(sink) in the denominator that
+    belongs to no key."""
+    m = scores.max() if sink is None else torch.maximum(scores.max(), torch.as_tensor(float(sink), dtype=F64))
+    e = torch.exp(scores - m)
+    return e / (e.sum() + (0.0 if sink is None else math.exp(float(sink) - float(m))))
 
 
 def capped(z, cap):
@@ -84,15 +81,15 @@ def attention(h, W, m):
     q = (h @ W("q").T).view(T, H, d)
     k = (h @ W("k").T).view(T, G, d)
     v = (h @ W("v").T).view(T, G, vd)
-    kr = [[rotate_halves(k[t, g], t, rd, base) for g in range(G)] for t in range(T)]
+    kr = torch.stack([torch.stack([rotate_halves(k[t, g], t, rd, base) for g in range(G)]) for t in range(T)])
     out = torch.zeros(T, H, vd, dtype=F64)
     for hh in range(H):
         g = hh // (H // G)
         for i in range(T):
             qi = rotate_halves(q[i, hh], i, rd, base)
-            lo, p = window_softmax(lambda j: capped((qi @ kr[j][g]) * scale, cap), i, win)
-            for n, j in enumerate(range(lo, i + 1)):
-                out[i, hh] += p[n] * v[j, g]
+            lo = max(0, i - win + 1) if win else 0  # the query sees itself and the win - 1 positions before it
+            p = window_softmax(capped((kr[lo:i + 1, g] @ qi) * scale, cap))
+            out[i, hh] = p @ v[lo:i + 1, g]
     return out.reshape(T, H * vd) @ W("o").T
 
 
@@ -125,9 +122,9 @@ def latent_attention(h, W, m, eps, rows):
         for i in range(T):
             qn = q[i, hh, :d]
             qr = rotate_adjacent(q[i, hh, d:], i, r, base)
-            lo, p = window_softmax(lambda j: (qn @ kh[j] + qr @ kr[j]) * scale, i, win, sink=sink[hh])
-            for n, j in enumerate(range(lo, i + 1)):
-                out[i, hh] += p[n] * vh[j]
+            lo = max(0, i - win + 1) if win else 0
+            p = window_softmax((kh[lo:i + 1] @ qn + kr[lo:i + 1] @ qr) * scale, sink=sink[hh])
+            out[i, hh] = p @ vh[lo:i + 1]
     gate = torch.sigmoid(h @ W("g").T)
     return (out.reshape(T, H * vd) * gate) @ W("o").T
 
