@@ -251,7 +251,8 @@ def case_window_edges(device, tol, dtype=torch.float32, bs=16, latent=False):
     visible keys instead, none of which carries the marker value), head 2 for the query's own position.  In a
     prompt's portion that follows cached context and for a decoded token; windows that end on, before and after
     page borders, pages out of order.  ``latent``: the values are the first columns of the key rows (one cache
-    tensor), and a sink far below the scores must change nothing."""
+    tensor); heads 0 and 2 carry a sink far below their scores, which must change nothing, head 1 a sink of 0 beside
+    its n visible keys of score 0, which must take exactly 1 / (n + 1) of the weight."""
     from githubrepostorag_amd.ops.attention import AttnMetadata, sink_attention
 
     dev = torch.device(device)
@@ -266,7 +267,7 @@ def case_window_edges(device, tol, dtype=torch.float32, bs=16, latent=False):
         for j in range(ctx):  # (latent: the value columns are key columns 0 .. vd - 1, so the markers sit at vd + j)
             kc[perm[j // bs], 0, j % bs, vd + j] = 30.0
             vc[perm[j // bs], 0, j % bs, 0] = j + 1.0  # the value names its position
-        sinks = torch.full((H,), -20.0, device=dev) if latent else None
+        sinks = torch.tensor([-20.0, 0.0, -20.0], device=dev) if latent else None
         for qlen in (33, 9, 1):  # (33 queries in bf16: the matrix-core kernel)
             q = torch.zeros(qlen, H, d)
             for n, p in enumerate(range(ctx - qlen, ctx)):
@@ -287,7 +288,20 @@ def case_window_edges(device, tol, dtype=torch.float32, bs=16, latent=False):
                 assert abs(float(got[n, 2, 0]) - (p + 1.0)) < tol * ctx, (window, qlen, p, "self")
                 if lo > 0:  # the key just outside gets nothing: head 1 sees a flat average of its window's values
                     want = float(torch.arange(lo, p + 1).double().mean()) + 1.0
+                    if latent:
+                        want *= (p + 1 - lo) / (p + 2 - lo)
                     assert abs(float(got[n, 1, 0]) - want) < tol * ctx, (window, qlen, p, "outside")
+            if latent:
+                continue
+            # a cap of 2 on the scores: the asked-for key scores 2 tanh(15) = 2, the other visible keys 0
+            got = sink_attention(q.to(dtype).to(dev), kc, vc, meta, 1.0, None, window=window,
+                                 softcap=2.0).float().cpu().view(qlen, H, vd)
+            e2 = float(np.exp(2.0))
+            for n, p in enumerate(range(ctx - qlen, ctx)):
+                lo = max(0, p - window + 1)
+                others = float(torch.arange(lo, p).double().sum()) + (p - lo)  # sum of (j + 1) over the keys before p
+                want = (e2 * (p + 1.0) + others) / (e2 + p - lo)
+                assert abs(float(got[n, 2, 0]) - want) < tol * ctx, (window, qlen, p, "capped")
 
 
 def case_generate(device, dtype=torch.float32, graphs=False, mixed=False, window=1, max_batched=4096, tol=2e-3,
